@@ -10,7 +10,8 @@
 // elements and values of dv, which need not be equal.  What a token computes depends on its position, window and cache content
 // only: not on the batch it is in nor on how its request was cut into steps.  Two options:
 // `slopes` (a value per query head) takes slope * (position - key position) off every score, and
-// `chunk` lets a token see only the keys of its own chunk of that many positions.
+// `chunk` lets a token see only the keys of its own chunk of that many positions; `sinks` (a value
+// per query head) adds exp(sink) to the softmax's denominator, a score that has no key or value.
 
 #include <hip/hip_runtime.h>
 
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     const T* __restrict__ v_cache, const int32_t* __restrict__ table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ slots, int nh, int nkv, int d, int dv, int page_size, int num_pages,
-    float scale, int window, const float* __restrict__ slopes, int chunk) {
+    float scale, int window, const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks) {
   __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
   __shared__ float p_s[kWavesPerBlock][kWave];
   __shared__ int64_t off_s[kWavesPerBlock][kWave];   // K row of each key of the tile
@@ -80,7 +81,13 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
   for (int i = lane; i < d; i += kWave) q_s[wave][i] = to_float(qh[i]);
   __syncthreads();
 
+  // a sink is a score with no key and no value that the denominator counts once: the running
+  // softmax starts from it instead of from nothing
   float m = -INFINITY, l = 0.f;
+  if (sinks != nullptr) {
+    m = sinks[h];
+    l = 1.f;
+  }
   float acc[kMaxHeadDim / kWave];
 #pragma unroll
   for (int i = 0; i < kMaxHeadDim / kWave; ++i) acc[i] = 0.f;
@@ -160,7 +167,8 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                                    const int32_t* positions, const int32_t* token_req,
                                    const int32_t* slots, int T, int nh, int nkv, int d, int dv,
                                    int page_size, int num_pages, float scale, int window,
-                                   const float* slopes, int chunk, int dtype, kvc_stream stream) {
+                                   const float* slopes, int chunk, const float* sinks, int dtype,
+                                   kvc_stream stream) {
   if (T < 0 || nh <= 0 || nkv <= 0 || page_size <= 0 || num_pages <= 0 || table_stride <= 0)
     return kvc_fail("kvc_paged_attention: bad sizes");
   if (nh % nkv) return kvc_fail("kvc_paged_attention: heads must be a multiple of kv heads");
@@ -179,7 +187,7 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                          static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
                          static_cast<const Tp*>(v_cache), table, table_stride, positions,
                          token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window, slopes,
-                         chunk));
+                         chunk, sinks));
   return kvc_check_launch("kvc_paged_attention");
 }
 

@@ -71,6 +71,7 @@ struct DecodeArgs {
   int window;
   const float* slopes;  // [nh] or null: slope * (position - key position) comes off the score
   int chunk;            // > 0: only the keys of the token's own chunk of so many positions
+  const float* sinks;   // [nh] or null: exp(sink) joins the softmax's denominator, with no key or value
   int nsplit;
   int lds_pages;  // page ids of a block's range that fit in LDS
 };
@@ -385,10 +386,12 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   for (int idx = tid; idx < g * D; idx += nthreads) {
     const int h = idx / D;
     const int e = idx - h * D;
-    float mmax = -INFINITY;
+    // the sink counts once for a row: the first split takes it, as one more partial sum without values
+    const float sink_l2e = (a.sinks != nullptr && split == 0) ? a.sinks[hk * g + h] * kLog2e : -INFINITY;
+    float mmax = sink_l2e;
     for (int w = 0; w < waves; ++w) mmax = fmaxf(mmax, sml[(w * 16 + h) * 2]);
     const float m_safe = (mmax == -INFINITY) ? 0.f : mmax;
-    float denom = 0.f, acc = 0.f;
+    float denom = __builtin_amdgcn_exp2f(sink_l2e - m_safe), acc = 0.f;
     for (int w = 0; w < waves; ++w) {
       const float wgt = __builtin_amdgcn_exp2f(sml[(w * 16 + h) * 2] - m_safe);
       if (wgt > 0.f) {
@@ -513,8 +516,8 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
                                     const int32_t* slots, const int32_t* token_rows,
                                     const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T, int nh,
                                     int nkv, int d, int page_size, int num_pages, float scale,
-                                    int window, const float* slopes, int chunk, int nsplit,
-                                    kvc_stream stream) {
+                                    int window, const float* slopes, int chunk, const float* sinks,
+                                    int nsplit, kvc_stream stream) {
   if (!kvc_decode_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_decode_attention: unsupported shape (bfloat16, head size a multiple of 32 "
                     "up to 256, at most 16 query heads per kv head, page size a multiple of 16)");
@@ -556,6 +559,7 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
   args.window = window;
   args.slopes = slopes;
   args.chunk = chunk;
+  args.sinks = sinks;
   args.nsplit = nsplit;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   kvc_note_variant(kVariantDecodeAttention, nsplit > 1 ? "decode_attention_kernel with splits" : "decode_attention_kernel");

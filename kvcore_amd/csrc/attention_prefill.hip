@@ -84,7 +84,8 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     const int32_t* __restrict__ table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int num_reqs, int nh,
     int nkv, int page_size, int num_pages, float scale_log2e, int window,
-    const float* __restrict__ slopes, int chunk, float* __restrict__ part_o, float* __restrict__ part_ml, int single,
+    const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int single,
     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim, int interleaved) {
   constexpr int kKeyBlocks = KB;
   constexpr int NJ = D / 16;
@@ -604,8 +605,20 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
 
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
-    const float l_row = quad_sum(l[ct]);
+    float l_row = quad_sum(l[ct]);
     if (!live[ct]) continue;
+    float m_l2e = (m[ct] == -INFINITY) ? -INFINITY : m[ct] * scale_log2e;  // the maximum in the exponent's units
+    if (sinks != nullptr && blockIdx.z == 0) {
+      // a sink is a score without key or value that the denominator counts once (in the first
+      // split): the row's sums move to the larger of their maximum and the sink
+      const float sink_l2e = sinks[my_head[ct]] * kLog2e;
+      const float top = fmaxf(m_l2e, sink_l2e);
+      const float keep = __builtin_amdgcn_exp2f(m_l2e - top);  // 0 when the row saw no key here
+      l_row = l_row * keep + __builtin_amdgcn_exp2f(sink_l2e - top);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) o_acc[ct][j] = o_acc[ct][j] * keep;
+      m_l2e = top;
+    }
     if (gridDim.z > 1) {
       // sums relative to m, and m in the exponent's units, as the combining kernel expects
       const int64_t slot =
@@ -614,7 +627,7 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
 #pragma unroll
       for (int j = 0; j < NJ; ++j) *reinterpret_cast<f32x4_t*>(po + 16 * j) = o_acc[ct][j];
       if (quad == 0) {
-        part_ml[2 * slot] = (m[ct] == -INFINITY) ? -INFINITY : m[ct] * scale_log2e;
+        part_ml[2 * slot] = m_l2e;
         part_ml[2 * slot + 1] = l_row;
       }
       continue;
@@ -636,7 +649,7 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
                       const bf16_t* v_cache, const int32_t* table, int table_stride,
                       const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                      const float* slopes, int chunk, float* part_o, float* part_ml, int nsplit, int single,
+                      const float* slopes, int chunk, const float* sinks, float* part_o, float* part_ml, int nsplit, int single,
                       const float* cos_tab,
                       const float* sin_tab, int rot_dim, int interleaved, hipStream_t stream) {
   const int g = nh / nkv;
@@ -665,7 +678,7 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB, W>), dim3(static_cast<unsigned>(wide), 1, nsplit), dim3(W * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, slopes, chunk,
-                     part_o, part_ml, single, cos_tab, sin_tab, rot_dim, interleaved);
+                     sinks, part_o, part_ml, single, cos_tab, sin_tab, rot_dim, interleaved);
   if (nsplit > 1) return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, stream);
   return kvc_check_launch("kvc_prefill_attention");
 }
@@ -675,7 +688,7 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    const bf16_t* v_cache, const int32_t* table, int table_stride,
                    const int32_t* positions, const int32_t* q_start, const int32_t* slots, int T,
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
-                   const float* slopes, int chunk, float* part_o, float* part_ml, int nsplit,
+                   const float* slopes, int chunk, const float* sinks, float* part_o, float* part_ml, int nsplit,
                    const float* cos_tab, const float* sin_tab,
                    int rot_dim, int interleaved, hipStream_t stream) {
   const int g = nh / nkv;
@@ -734,7 +747,7 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
 #define KVC_LAUNCH_PREFILL(CT_, W_)                                                                      \
   return launch_prefill_ct<D, CT_, W_>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions, \
                                        q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window, \
-                                       slopes, chunk, part_o, part_ml, nsplit, single, cos_tab, sin_tab, rot_dim,     \
+                                       slopes, chunk, sinks, part_o, part_ml, nsplit, single, cos_tab, sin_tab, rot_dim,     \
                                        interleaved, stream)
   if (waves == 8) {
     if (ct == 2) KVC_LAUNCH_PREFILL(2, 8);
@@ -760,7 +773,7 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
                                      const int32_t* positions, const int32_t* q_start,
                                      const int32_t* slots, int T, int R, int nh, int nkv, int d,
                                      int page_size, int num_pages, float scale, int window,
-                                     const float* slopes, int chunk, void* part_o, void* part_ml, int nsplit, const float* cos_tab,
+                                     const float* slopes, int chunk, const float* sinks, void* part_o, void* part_ml, int nsplit, const float* cos_tab,
                                      const float* sin_tab, int rot_dim, int interleaved,
                                      kvc_stream stream) {
   if (!kvc_prefill_attention_supported(nh, nkv, d, page_size, 1))
@@ -790,8 +803,8 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
   if (d == 64)
     return launch_prefill<64>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                               positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                              window, slopes, chunk, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
+                              window, slopes, chunk, sinks, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
   return launch_prefill<128>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                              positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                             window, slopes, chunk, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
+                             window, slopes, chunk, sinks, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
 }

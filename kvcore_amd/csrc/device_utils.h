@@ -48,6 +48,15 @@ __device__ __forceinline__ float rotate_second(float x0, float x1, float c, floa
   return __builtin_fmaf(x0, s, x1 * c);
 }
 
+// The activation of a gated feed-forward's gate: kGateSilu g * sigmoid(g), kGateGeluTanh the tanh
+// form of gelu, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
+constexpr int kGateSilu = 0;
+constexpr int kGateGeluTanh = 1;
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == kGateGeluTanh) return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.f + expf(-g));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

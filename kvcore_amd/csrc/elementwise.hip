@@ -442,7 +442,7 @@ extern "C" int kvc_residual_add2(float* residual, const void* a, int a_dtype, co
 
 template <typename T>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int I,
-                                int64_t n) {
+                                int64_t n, int act) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const int64_t t = idx / I;
@@ -450,13 +450,12 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gate_
   const T* row = gate_up + t * 2 * I;
   const float g = to_float(row[i]);
   const float u = to_float(row[I + i]);
-  const float s = g / (1.f + expf(-g));
-  out[idx] = from_float<T>(s * u);
+  out[idx] = from_float<T>(gate_act(g, act) * u);
 }
 
 template <typename T>
 __global__ void silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gate_up, int I8,
-                                    int64_t n8) {
+                                    int64_t n8, int act) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= n8) return;
   const int64_t t = idx / I8;
@@ -466,13 +465,19 @@ __global__ void silu_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ g
   load8(gate_up + t * 2 * I + i, g);
   load8(gate_up + t * 2 * I + I + i, u);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) y[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+  for (int e = 0; e < 8; ++e) y[e] = gate_act(g[e], act) * u[e];
   store8(out + t * I + i, y);
 }
 
 extern "C" int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype,
                             kvc_stream stream) {
-  if (T < 0 || I <= 0) return kvc_fail("kvc_silu_mul: bad sizes");
+  return kvc_gate_mul(out, gate_up, T, I, kGateSilu, dtype, stream);
+}
+
+extern "C" int kvc_gate_mul(void* out, const void* gate_up, int T, int I, int act, int dtype,
+                            kvc_stream stream) {
+  if (T < 0 || I <= 0) return kvc_fail("kvc_gate_mul: bad sizes");
+  if (act != kGateSilu && act != kGateGeluTanh) return kvc_fail("kvc_gate_mul: unknown activation");
   const int64_t n = static_cast<int64_t>(T) * I;
   if (n == 0) return 0;
   if (I % 8 == 0 && (reinterpret_cast<uintptr_t>(out) % 16) == 0 &&
@@ -482,15 +487,15 @@ extern "C" int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dt
     KVC_DISPATCH_DTYPE(dtype, Tp,
                        hipLaunchKernelGGL(silu_mul_vec_kernel<Tp>, dim3(vblocks), dim3(256), 0,
                                           S(stream), static_cast<Tp*>(out),
-                                          static_cast<const Tp*>(gate_up), I / 8, n8));
-    return kvc_check_launch("kvc_silu_mul");
+                                          static_cast<const Tp*>(gate_up), I / 8, n8, act));
+    return kvc_check_launch("kvc_gate_mul");
   }
   const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
   KVC_DISPATCH_DTYPE(dtype, Tp,
                      hipLaunchKernelGGL(silu_mul_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),
                                         static_cast<Tp*>(out), static_cast<const Tp*>(gate_up), I,
-                                        n));
-  return kvc_check_launch("kvc_silu_mul");
+                                        n, act));
+  return kvc_check_launch("kvc_gate_mul");
 }
 
 // ----------------------------------------------------------------------- row gather

@@ -49,7 +49,7 @@ template <int WAVES, int RT, int NT, bool GATED, typename OutT>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
     OutT* __restrict__ C, float* __restrict__ partial, const bf16_t* __restrict__ A,
     const bf16_t* __restrict__ W, const bf16_t* __restrict__ bias, int M, int N, int K, int64_t lda,
-    int64_t ldc, int k_per_block, int packed) {
+    int64_t ldc, int k_per_block, int packed, int act) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   static_assert(kStages % (2 * kChunkSteps) == 0, "a round of stages must cover whole pairs of chunks");
   __shared__ __attribute__((aligned(16))) bf16_t a_lds[2][NT * 16 * kRowElems];
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mid_kernel(
       for (int i = 0; i < 4; ++i) {
         const float gv = to_float(from_float<bf16_t>(acc[0][nt][i] + bg[i]));
         const float uv = to_float(from_float<bf16_t>(acc[1][nt][i] + bu[i]));
-        y[i] = gv / (1.f + expf(-gv)) * uv;
+        y[i] = gate_act(gv, act) * uv;
       }
       store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, y, n_left);
     }
@@ -274,6 +274,7 @@ struct MidPlan {
   int slices;  // along K
   int k_per_block;
   int packed;  // W is in kvc_pack_weight's order
+  int act;     // the gate's activation in the gated form (kGateSilu, kGateGeluTanh)
 };
 
 // Blocks enough for every compute unit, from N and K alone.  Narrow outputs are cut along K
@@ -282,6 +283,7 @@ struct MidPlan {
 MidPlan plan_mid(int N, int K, bool gated, bool may_slice) {
   MidPlan p;
   p.packed = 0;
+  p.act = kGateSilu;
   // two waves a block where four would leave compute units without one
   p.waves = (gated && (N + 63) / 64 < 192) ? 2 : 4;
   p.rt = gated ? 2 : (N >= 16384 ? 2 : 1);
@@ -314,7 +316,7 @@ void launch_mid(OutT* C, float* partial, const bf16_t* A, const bf16_t* W, const
   const int cols_per_block = WAVES * (GATED ? 16 : 16 * RT);
   const dim3 grid((N + cols_per_block - 1) / cols_per_block, p.slices), block(WAVES * 64);
   hipLaunchKernelGGL((gemm_mid_kernel<WAVES, RT, NT, GATED, OutT>), grid, block, 0, stream, C,
-                     p.slices > 1 ? partial : nullptr, A, W, bias, M, N, K, lda, ldc, p.k_per_block, p.packed);
+                     p.slices > 1 ? partial : nullptr, A, W, bias, M, N, K, lda, ldc, p.k_per_block, p.packed, p.act);
 }
 
 template <bool GATED, typename OutT>
@@ -382,17 +384,18 @@ extern "C" int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const vo
                                  int packed, kvc_stream stream) {
   if (int rc = check_mid(A, W, M, N, K, lda, ldc)) return rc;
   if (packed && N % 16) return kvc_fail("kvc_gemm_mid_bf16: packed weights have a multiple of 16 rows");
-  if (mode < 0 || mode > 3) return kvc_fail("kvc_gemm_mid_bf16: unknown mode");
+  if (mode < 0 || mode > 4) return kvc_fail("kvc_gemm_mid_bf16: unknown mode");
   if (M == 0) return 0;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bf16_t* a = static_cast<const bf16_t*>(A);
   const bf16_t* w = static_cast<const bf16_t*>(W);
   const bf16_t* b = static_cast<const bf16_t*>(bias);
   float* part = static_cast<float*>(partial);
-  if (mode == 1) {  // silu(A Wg^T) * (A Wu^T): one slice, bfloat16
+  if (mode == 1 || mode == 4) {  // act(A Wg^T) * (A Wu^T): one slice, bfloat16; 1 silu, 4 gelu (tanh form)
     if (out_dtype != 1) return kvc_fail("kvc_gemm_mid_bf16: the gated form stores bfloat16");
     MidPlan p = plan_mid(N, K, true, false);
     p.packed = packed;
+    p.act = mode == 4 ? kGateGeluTanh : kGateSilu;
     return dispatch_mid<true>(static_cast<bf16_t*>(C), nullptr, a, w, b, M, N, K, lda, ldc, p, s);
   }
   if (mode == 2) {  // only the slices' partial sums

@@ -42,6 +42,7 @@ struct SkinnyExtras {
   int64_t ldr;
   const float* gain;
   float* out_ss;
+  int act;  // the gate's activation in the gated form (kGateSilu, kGateGeluTanh)
 };
 
 // GATED: the two row tiles of a wave are rows n of the first N weight rows (gate) and rows
@@ -317,7 +318,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
       for (int i = 0; i < 4; ++i) {
         const float gv = to_float(from_float<bf16_t>(acc[0][nt][i] * row_scale[nt] + bg[i]));
         const float uv = to_float(from_float<bf16_t>(acc[1][nt][i] * row_scale[nt] + bu[i]));
-        y[i] = gv / (1.f + expf(-gv)) * uv;
+        y[i] = gate_act(gv, ex.act) * uv;
       }
       store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, y, n_left);
     }
@@ -515,7 +516,7 @@ int check_operands(const char* who, const void* A, const void* W, int M, int N, 
   return 0;
 }
 
-const SkinnyExtras kNoExtras = {nullptr, 0, 1.f, 0.f, nullptr, 0, nullptr, nullptr};
+const SkinnyExtras kNoExtras = {nullptr, 0, 1.f, 0.f, nullptr, 0, nullptr, nullptr, kGateSilu};
 
 }  // namespace
 
@@ -597,8 +598,9 @@ extern "C" int kvc_gemm_skinny_fused_bf16(void* C, const void* A, const void* W,
     return kvc_fail("kvc_gemm_skinny_fused_bf16: the residual form needs gain and out_ss, rows of "
                     "at least N, and is not gated");
   if (M == 0) return 0;
+  if (gated < 0 || gated > 2) return kvc_fail("kvc_gemm_skinny_fused_bf16: gated is 0, 1 (silu) or 2 (gelu, tanh form)");
   SkinnyExtras ex = {in_ss, in_parts, static_cast<float>(in_width), in_eps,
-                     residual, ldr, gain, out_ss};
+                     residual, ldr, gain, out_ss, gated == 2 ? kGateGeluTanh : kGateSilu};
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (gated)
     return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),

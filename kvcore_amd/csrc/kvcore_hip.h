@@ -82,6 +82,9 @@ int kvc_residual_add2(float* residual, const void* a, int a_dtype, const void* b
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i].
 int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype, kvc_stream stream);
+// out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]; act 0: silu, 1: gelu in its tanh form,
+// 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
+int kvc_gate_mul(void* out, const void* gate_up, int T, int I, int act, int dtype, kvc_stream stream);
 
 // out[s, :] = in[rows[s], :]; `in` may be float32 (in_dtype 0) while out is dt.
 int kvc_gather_rows(void* out, const void* in, const int32_t* rows, int S, int H, int in_dtype,
@@ -118,13 +121,15 @@ int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_
 // q is [T, nh, d] with q_stride elements between tokens; keys have d elements, values dv (K
 // pages [kv head, page_size, d], V pages [kv head, dv, page_size]); out is [T, nh*dv].
 // slopes (float32 [nh], or null): slopes[h] * (p - key position) is taken off every score of head
-// h.  chunk > 0: a token sees only the keys j with j / chunk == p / chunk.
+// h.  chunk > 0: a token sees only the keys j with j / chunk == p / chunk.  sinks (float32 [nh],
+// or null): exp(sinks[h]) is added to the softmax's denominator of head h, a score that has no
+// key and no value and is not scaled.
 int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                         const void* v_cache, const int32_t* table, int table_stride,
                         const int32_t* positions, const int32_t* token_req,
                         const int32_t* slots, int T, int nh, int nkv, int d, int dv, int page_size,
                         int num_pages, float scale, int window, const float* slopes, int chunk,
-                        int dtype, kvc_stream stream);
+                        const float* sinks, int dtype, kvc_stream stream);
 
 // What kvc_rope_kv_write does, for heads whose keys (d) and values (dv) may differ in size,
 // with a norm of every q and k head before the rotation: rows of qkv are [nh q heads of d |
@@ -212,6 +217,7 @@ int kvc_gated_group_rmsnorm(void* out, int out_dtype, const float* y, const void
 // Per head h (its q and k come from head h / (nh / nqk) of nqk heads of d), token by token:
 //   delta_rule 0:  S = diag(decay[t, h, :]) S + k v^T            (decay rows of nh * d values)
 //   delta_rule 1:  S = decay[t, h] S;  u = beta[t, h] (v - S^T k);  S = S + k u^T
+//   delta_rule 2:  S = decay[t, h] S + beta[t, h] k v^T          (scalar gates per head)
 // and out[t, h] = S^T (q_scale q) after the token's write; out is [T, nh * dv] float32.  q, k, v, decay and
 // beta are float32 rows with strides.  d at most 256.
 int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const float* k,
@@ -220,6 +226,23 @@ int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const fl
                           const int32_t* positions, const int32_t* token_req, const int32_t* q_start,
                           const int32_t* slots, int R, int nh, int nqk, int d, int dv, int delta_rule,
                           float q_scale, kvc_stream stream);
+// The gates of a matrix memory with log gates and a running maximum m (mLSTM), per request in
+// token order: i = cap tanh((i_raw + i_bias) / cap), f = logsigmoid(cap tanh((f_raw + f_bias) / cap)),
+// m_t = max(f + m_(t-1), i), keep[t, h] = exp(f + m_(t-1) - m_t), take[t, h] = exp(i - m_t),
+// m_out[t, h] = m_t; m is 0 before position 0, else m_state[slot, h], which receives the last m.
+// keep, take, m_out are [T, nh] float32; i_raw and f_raw float32 rows with strides.
+int kvc_max_gates(float* keep, float* take, float* m_out, const float* i_raw, int64_t i_stride,
+                  const float* f_raw, int64_t f_stride, const float* i_bias, const float* f_bias,
+                  float cap, float* m_state, const int32_t* positions, const int32_t* token_req,
+                  const int32_t* q_start, const int32_t* slots, int R, int nh, kvc_stream stream);
+// out[t, h, c] = y / sqrt(mean_c y^2 + eps) * gain[h * dv + c] * sigmoid(gate[t, h, c]) with
+// y = o[t, h, c] / (max(|o[t, h, dv]|, exp(-m[t, h])) + den_eps); o is [T, heads, dv + 1] float32.
+int kvc_max_gated_finish(void* out, int out_dtype, const float* o, const float* m, const void* gate,
+                         int64_t gate_stride, int gate_dtype, const float* gain, float eps,
+                         float den_eps, int T, int heads, int dv, kvc_stream stream);
+// out[t, h, :dv] = v[t, h, :], out[t, h, dv] = 1; out is [T, heads, dv + 1] float32.
+int kvc_append_ones(float* out, const float* v, int64_t v_stride, int T, int heads, int dv,
+                    kvc_stream stream);
 // a[t, i] = sigmoid(z[t, i] + bias[i]) ^ inv_tau, computed as exp(inv_tau * log sigmoid); bias may be null.
 int kvc_sigmoid_power(float* a, const float* z, int64_t z_stride, const float* bias, float inv_tau,
                       int T, int W, kvc_stream stream);
@@ -286,7 +309,7 @@ int kvc_clamped_glu(void* out, const void* gate_up, int T, int I, float limit, f
 // kvc_decode_attention_max_table: the widest block table (entries per request) whose page ids
 // for one split still fit in a block's LDS; a wider one is refused, so engines check it when
 // they are built.
-// slopes (float32 [nh] or null) and chunk as for kvc_paged_attention; the kernel for portions
+// slopes, sinks (float32 [nh] or null) and chunk as for kvc_paged_attention; the kernel for portions
 // (kvc_prefill_attention) takes them too.
 int kvc_decode_attention_supported(int nh, int nkv, int d, int page_size, int dtype);
 int kvc_decode_attention_waves(int nh, int nkv, int d);
@@ -297,7 +320,8 @@ int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv
                          const int32_t* slots, const int32_t* token_rows, const float* cos_tab,
                          const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T,
                          int nh, int nkv, int d, int page_size, int num_pages, float scale,
-                         int window, const float* slopes, int chunk, int nsplit, kvc_stream stream);
+                         int window, const float* slopes, int chunk, const float* sinks, int nsplit,
+                         kvc_stream stream);
 
 // The same attention for bfloat16 portions of prompts on the matrix cores: a block per
 // (tile of a request's tokens, kv head), keys staged through LDS.  q_start [R+1] bounds
@@ -313,9 +337,29 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
                           const void* v_cache, const int32_t* table, int table_stride,
                           const int32_t* positions, const int32_t* q_start, const int32_t* slots,
                           int T, int R, int nh, int nkv, int d, int page_size, int num_pages,
-                          float scale, int window, const float* slopes, int chunk, void* part_o, void* part_ml, int nsplit,
+                          float scale, int window, const float* slopes, int chunk, const float* sinks, void* part_o,
+                          void* part_ml, int nsplit,
                           const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved,
                           kvc_stream stream);
+
+// ---- norms after a sublayer, norms over a whole projection, gates per head (norm_ops.hip)
+// residual[t, :] += post_gain * delta[t, :] / sqrt(mean(delta[t, :]^2) + eps), and then, if out is
+// not null, out[t, :] = next_gain * residual[t, :] / sqrt(mean(residual[t, :]^2) + next_eps): the norm
+// behind a sublayer, the sum into the float32 stream and the norm before the next sublayer in one
+// pass.  delta is float32 (delta_dtype 0) or bfloat16 (1); out likewise (out_dtype).
+int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* delta, int delta_dtype,
+                      const float* post_gain, float eps, const float* next_gain, float next_eps,
+                      int T, int H, kvc_stream stream);
+// Rows of qkv are [nq | nk | ...]: the first nq values (all query heads at once) are divided by
+// their root mean square (eps inside the root) and multiplied by q_gain [nq], the next nk values
+// likewise with k_gain [nk], in place; with copy_k the nk values as they were before the norm
+// are copied behind them first (values that are the keys as projected).
+int kvc_wide_qk_norm(void* qkv, int64_t stride, const float* q_gain, const float* k_gain, float eps,
+                     int T, int nq, int nk, int copy_k, int dtype, kvc_stream stream);
+// out[t, h * n + e] = x[t * x_stride + h * head_stride + skip + e] * sigmoid(gate[t * gate_stride + h]),
+// e < n: a gate per head, and a run of each head's columns kept.  gate has the dtype of x and out.
+int kvc_head_gate(void* out, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,
+                  int T, int heads, int head_stride, int skip, int n, int dtype, kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) in float32 with float32 products and sums;
 // each element is one running sum over k = 0..K-1, whatever M is.
@@ -325,7 +369,7 @@ int kvc_gemm_f32(float* C, const float* A, const float* W, const float* bias, in
 // The same product for 17 to 192 rows, where the waves of a block share the rows of A through
 // LDS (K a multiple of 512).  mode 0: C = A W^T (+ bias), float32 (out_dtype 0) or bfloat16
 // (1).  mode 1: C[M, N] = silu(A Wg^T + bg) * (A Wu^T + bu) in bfloat16, W [2N, K] holding Wg
-// then Wu.  mode 2: narrow outputs are cut along K into kvc_gemm_mid_slices(N, K) slices and
+// then Wu (mode 4: the same with the tanh form of gelu for silu).  mode 2: narrow outputs are cut along K into kvc_gemm_mid_slices(N, K) slices and
 // only their float32 partial sums are stored, partial [slices, M, N] (no bias); the kernel
 // that consumes them adds them up in slice order.  mode 3: as mode 0, but cut along K like
 // mode 2 when `partial` is given, with a second kernel that sums the slices.  With `packed` W

@@ -4,7 +4,8 @@
 // kvc_linear_state_scan walks each request's tokens in order.  Two update rules:
 //   key decay   S <- diag(a_t) S + k_t v_t^T                      (a_t one factor per key channel)
 //   delta rule  S <- g_t S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T   (g_t, beta_t scalars)
-// and in both o_t = S^T (q_scale q_t), read after the token's write.  A block owns one (request, head, tile
+//   scalar gates  S <- g_t S + beta_t k_t v_t^T                   (g_t, beta_t scalars per head)
+// and in all o_t = S^T (q_scale q_t), read after the token's write.  A block owns one (request, head, tile
 // of VT value channels); the NSL threads that share a column of the state are neighbouring lanes
 // (their partial sums meet through lane permutations, in one fixed order) and each keeps NPT rows in
 // registers; q, k, the factors and v of 16 tokens at a time go through LDS.  A request whose
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     int64_t decay_stride, const float* __restrict__ beta, int64_t beta_stride, float* __restrict__ state,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int nqk, int d,
-    int dv, float q_scale) {
+    int dv, float q_scale, int scalar_gates) {
   constexpr int VT = 256 / NSL;  // value channels a block
   // FULL: d == NPT * NSL, so no row needs a bound, and a thread's rows of q, k and the factors lie
   // side by side in LDS (row n of a token at (n % NSL) * NPT + n / NSL), read 16 bytes at a time
@@ -114,7 +115,23 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       constexpr int ST = FULL ? 1 : NSL;  // from one of the thread's rows to its next, in LDS
       const float vv = v_s[tt * VT + pl];
       float acc = 0.f;
-      if (DELTA) {
+      if (DELTA && scalar_gates) {  // the same for the whole grid: S <- g S + (beta k) v^T
+        const float g = a_s[2 * tt], bv = a_s[2 * tt + 1] * vv;
+        float acc1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NPT; i += 2) {
+          const int n = ns + NSL * i;
+          if (FULL || n < d) {
+            s[i] = fmaf(g, s[i], kt[ST * i] * bv);
+            acc = fmaf(s[i], qt[ST * i], acc);
+          }
+          if (FULL || n + NSL < d) {
+            s[i + 1] = fmaf(g, s[i + 1], kt[ST * (i + 1)] * bv);
+            acc1 = fmaf(s[i + 1], qt[ST * (i + 1)], acc1);
+          }
+        }
+        acc += acc1;
+      } else if (DELTA) {
         const float g = a_s[2 * tt], bt = a_s[2 * tt + 1];
         float kd0 = 0.f, kd1 = 0.f;  // two running sums: half as long a chain of dependent operations
 #pragma unroll
@@ -336,7 +353,156 @@ __global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(
     op[i] = from_float<TO>(p[i] * inv * gain[i] * silu_ff(to_float(gp[i])));
 }
 
+
+// The log gates of a matrix memory with a running maximum (mLSTM), for every request's tokens in
+// order: i = cap tanh((i_raw + bi) / cap), f = logsigmoid(cap tanh((f_raw + bf) / cap)),
+// m_t = max(f_t + m_(t-1), i_t), keep_t = exp(f_t + m_(t-1) - m_t), take_t = exp(i_t - m_t).
+// A block a request: the gates of all its tokens side by side, then a thread a head walks the
+// maxima in order (an addition and a maximum a token), then the exponentials side by side.
+// m starts at 0 at position 0 and otherwise comes from the slot's state, where it goes back.
+__global__ __launch_bounds__(256) void max_gates_kernel(
+    float* __restrict__ keep, float* __restrict__ take, float* __restrict__ m_out, const float* __restrict__ i_raw,
+    int64_t i_stride, const float* __restrict__ f_raw, int64_t f_stride, const float* __restrict__ i_bias,
+    const float* __restrict__ f_bias, float cap, float* __restrict__ m_state, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ token_req, const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots,
+    int nh) {
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const int b = q_start[r], e = q_start[r + 1];
+  if (e <= b) return;
+  const int n = (e - b) * nh;
+  if (token_req[b] < 0) {  // padding rows
+    for (int idx = tid; idx < n; idx += blockDim.x) {
+      keep[static_cast<int64_t>(b) * nh + idx] = 0.f;
+      take[static_cast<int64_t>(b) * nh + idx] = 0.f;
+      m_out[static_cast<int64_t>(b) * nh + idx] = 0.f;
+    }
+    return;
+  }
+  const float inv_cap = 1.f / cap;
+  for (int idx = tid; idx < n; idx += blockDim.x) {
+    const int tt = idx / nh, h = idx - tt * nh;
+    const int64_t t = b + tt;
+    const float gi = cap * tanhf((i_raw[t * i_stride + h] + i_bias[h]) * inv_cap);
+    const float gf = log_sigmoid_f(cap * tanhf((f_raw[t * f_stride + h] + f_bias[h]) * inv_cap));
+    take[t * nh + h] = gi;  // the log gates, until the maxima are known
+    keep[t * nh + h] = gf;
+  }
+  __syncthreads();
+  float* ms = m_state + static_cast<int64_t>(slots[r]) * nh;
+  const bool fresh = positions[b] == 0;
+  for (int h = tid; h < nh; h += blockDim.x) {
+    float m = fresh ? 0.f : ms[h];
+    for (int64_t t = b; t < e; ++t) {
+      // the maximum before this token goes where the token's own will stand: m_out[t] holds
+      // m_(t-1) until the pass below has read it
+      const float gf = keep[t * nh + h], gi = take[t * nh + h];
+      m_out[t * nh + h] = m;
+      m = fmaxf(gf + m, gi);
+    }
+    ms[h] = m;
+  }
+  __syncthreads();
+  for (int idx = tid; idx < n; idx += blockDim.x) {
+    const int64_t at = static_cast<int64_t>(b) * nh + idx;
+    const float gf = keep[at], gi = take[at], before = m_out[at];
+    const float m = fmaxf(gf + before, gi);  // the same operations as the walk's, so the same bits
+    keep[at] = expf(gf + before - m);
+    take[at] = expf(gi - m);
+    m_out[at] = m;
+  }
+}
+
+// The end of the same mixer: o[t, h, :dv] and the normaliser's product with the query at column dv
+// of each head's dv + 1 columns.  y = o / (max(|n.q|, exp(-m)) + den_eps); y over its root mean
+// square (eps inside the root) times gain[h * dv + c] times sigmoid(gate[t, h, c]).  A wave a
+// (token, head).
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void max_gated_finish_kernel(
+    TO* __restrict__ out, const float* __restrict__ o, const float* __restrict__ m, const TG* __restrict__ gate,
+    int64_t gate_stride, const float* __restrict__ gain, float eps, float den_eps, int T, int heads, int dv) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (item >= static_cast<int64_t>(T) * heads) return;
+  const int t = static_cast<int>(item / heads), h = static_cast<int>(item - static_cast<int64_t>(t) * heads);
+  const float* p = o + item * (dv + 1);
+  const TG* gp = gate + t * gate_stride + static_cast<int64_t>(h) * dv;
+  const float den = fmaxf(fabsf(p[dv]), expf(-m[item])) + den_eps;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += kWave) {
+    const float y = p[i] / den;
+    ss = fmaf(y, y, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(dv) + eps);
+  TO* op = out + item * dv;
+  const float* gn = gain + static_cast<int64_t>(h) * dv;
+  for (int i = lane; i < dv; i += kWave)
+    op[i] = from_float<TO>(p[i] / den * inv * gn[i] * sigmoid_f(to_float(gp[i])));
+}
+
+// v_out[t, h, :dv] = v[t, h, :], v_out[t, h, dv] = 1: the values with a column of ones, whose
+// column of the state is the normaliser.
+__global__ __launch_bounds__(256) void append_ones_kernel(float* __restrict__ out, const float* __restrict__ v,
+                                                          int64_t v_stride, int T, int heads, int dv) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int w = dv + 1;
+  if (idx >= static_cast<int64_t>(T) * heads * w) return;
+  const int64_t th = idx / w;
+  const int c = static_cast<int>(idx - th * w);
+  const int64_t t = th / heads;
+  const int h = static_cast<int>(th - t * heads);
+  out[idx] = c < dv ? v[t * v_stride + static_cast<int64_t>(h) * dv + c] : 1.f;
+}
+
 }  // namespace
+
+extern "C" int kvc_max_gates(float* keep, float* take, float* m_out, const float* i_raw, int64_t i_stride,
+                             const float* f_raw, int64_t f_stride, const float* i_bias, const float* f_bias,
+                             float cap, float* m_state, const int32_t* positions, const int32_t* token_req,
+                             const int32_t* q_start, const int32_t* slots, int R, int nh, kvc_stream stream) {
+  if (R < 0 || nh <= 0 || i_stride < nh || f_stride < nh || !(cap > 0.f)) return kvc_fail("kvc_max_gates: bad sizes");
+  if (R == 0) return 0;
+  hipLaunchKernelGGL(max_gates_kernel, dim3(R), dim3(256), 0, S(stream), keep, take, m_out, i_raw, i_stride, f_raw,
+                     f_stride, i_bias, f_bias, cap, m_state, positions, token_req, q_start, slots, nh);
+  return kvc_check_launch("kvc_max_gates");
+}
+
+extern "C" int kvc_max_gated_finish(void* out, int out_dtype, const float* o, const float* m, const void* gate,
+                                    int64_t gate_stride, int gate_dtype, const float* gain, float eps,
+                                    float den_eps, int T, int heads, int dv, kvc_stream stream) {
+  if (T < 0 || heads <= 0 || dv <= 0 || gate_stride < static_cast<int64_t>(heads) * dv)
+    return kvc_fail("kvc_max_gated_finish: bad sizes");
+  if (T == 0) return 0;
+  const int64_t waves = static_cast<int64_t>(T) * heads;
+  const dim3 grid(static_cast<unsigned>((waves + 3) / 4));
+#define KVC_MGF(TG, TO)                                                                                        \
+  hipLaunchKernelGGL((max_gated_finish_kernel<TG, TO>), grid, dim3(256), 0, S(stream), static_cast<TO*>(out), o, m, \
+                     static_cast<const TG*>(gate), gate_stride, gain, eps, den_eps, T, heads, dv)
+  if (gate_dtype == 0 && out_dtype == 0) {
+    KVC_MGF(float, float);
+  } else if (gate_dtype == 0 && out_dtype == 1) {
+    KVC_MGF(float, bf16_t);
+  } else if (gate_dtype == 1 && out_dtype == 1) {
+    KVC_MGF(bf16_t, bf16_t);
+  } else if (gate_dtype == 1 && out_dtype == 0) {
+    KVC_MGF(bf16_t, float);
+  } else {
+    return kvc_fail("kvc_max_gated_finish: unknown dtype code");
+  }
+#undef KVC_MGF
+  return kvc_check_launch("kvc_max_gated_finish");
+}
+
+extern "C" int kvc_append_ones(float* out, const float* v, int64_t v_stride, int T, int heads, int dv,
+                               kvc_stream stream) {
+  if (T < 0 || heads <= 0 || dv <= 0 || v_stride < static_cast<int64_t>(heads) * dv)
+    return kvc_fail("kvc_append_ones: bad sizes");
+  if (T == 0) return 0;
+  const int64_t n = static_cast<int64_t>(T) * heads * (dv + 1);
+  hipLaunchKernelGGL(append_ones_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, S(stream), out, v,
+                     v_stride, T, heads, dv);
+  return kvc_check_launch("kvc_append_ones");
+}
 
 extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const float* k,
                                      int64_t k_stride, const float* v, int64_t v_stride,
@@ -344,11 +510,15 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
                                      int64_t beta_stride, float* state, const int32_t* positions,
                                      const int32_t* token_req, const int32_t* q_start,
                                      const int32_t* slots, int R, int nh, int nqk, int d, int dv,
-                                     int delta_rule, float q_scale, kvc_stream stream) {
+                                     int rule, float q_scale, kvc_stream stream) {
+  if (rule < 0 || rule > 2) return kvc_fail("kvc_linear_state_scan: the rule is 0 (key decay), 1 (delta) or 2 (scalar gates)");
+  const int delta_rule = rule != 0;  // a gate and a factor per head and token instead of a decay per key channel
+  const int scalar_gates = rule == 2;
   if (R < 0 || nh <= 0 || nqk <= 0 || nh % nqk || d <= 0 || dv <= 0)
     return kvc_fail("kvc_linear_state_scan: bad sizes");
   if (d > 256) return kvc_fail("kvc_linear_state_scan: at most 256 key channels a head");
-  if (delta_rule && beta == nullptr) return kvc_fail("kvc_linear_state_scan: the delta rule needs beta");
+  if (delta_rule && beta == nullptr) return kvc_fail("kvc_linear_state_scan: this rule needs beta");
+  if (delta_rule && beta_stride < nh) return kvc_fail("kvc_linear_state_scan: rows of beta too short for the heads");
   if (q_stride < static_cast<int64_t>(nqk) * d || k_stride < static_cast<int64_t>(nqk) * d ||
       v_stride < static_cast<int64_t>(nh) * dv || decay_stride < (delta_rule ? nh : static_cast<int64_t>(nh) * d))
     return kvc_fail("kvc_linear_state_scan: rows too short for the heads");
@@ -367,7 +537,7 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_, FULL_, PF_>), grid, dim3(256),               \
                      lds*(PF_ ? 2 : 1), S(stream), out, q, q_stride, k, k_stride, v, v_stride, decay,         \
                      decay_stride, beta, beta_stride, state, positions, token_req, q_start, slots, nh, nqk, d, \
-                     dv, q_scale)
+                     dv, q_scale, scalar_gates)
   // two sets of LDS buffers (the next stage fetched while one is worked on) where a stage's values
   // deal out evenly to the threads and both sets fit the 64 KB a block may take
 #define KVC_LSCAN(NPT, DELTA, NSL_)                                                  \

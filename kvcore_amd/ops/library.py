@@ -42,12 +42,19 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_residual_add": [P, P, I, I, I, P],
         "kvc_residual_add2": [P, P, I, P, I, I, I, P],
         "kvc_silu_mul": [P, P, I, I, I, P],
+        "kvc_gate_mul": [P, P, I, I, I, I, P],
+        "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, P],
+        "kvc_wide_qk_norm": [P, L, P, P, F, I, I, I, I, I, P],
+        "kvc_head_gate": [P, P, L, P, L, I, I, I, I, I, I, P],
+        "kvc_max_gates": [P, P, P, P, L, P, L, P, P, F, P, P, P, P, P, I, I, P],
+        "kvc_max_gated_finish": [P, I, P, P, P, L, I, P, F, F, I, I, I, P],
+        "kvc_append_ones": [P, P, L, I, I, I, P],
         "kvc_gather_rows": [P, P, P, I, I, I, I, P],
         "kvc_to_float": [P, P, L, I, P],
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
-        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, I, P],
+        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, I, P],
         "kvc_linear_state_scan": [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, P],
         "kvc_sigmoid_power": [P, P, L, P, F, I, I, P],
         "kvc_decay_and_write_gates": [P, P, P, L, P, L, P, P, I, I, P],
@@ -72,11 +79,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_ssm_scan": [P, P, L, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "kvc_gated_group_rmsnorm": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
-                                 F, I, P, I, I, P],
+                                 F, I, P, I, P, I, P],
         "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_max_table": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
-        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, P, I,
+        "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, P, P, I,
                                   P, P, I, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_mid_slices": [I, I],
@@ -277,12 +284,23 @@ def residual_add2(residual: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> N
                                     _dev(b, "b"), _code(b, "b"), T, H, _stream()), "kvc_residual_add2")
 
 
-def silu_mul(out: torch.Tensor, gate_up: torch.Tensor) -> None:
+GATE_ACTS = {"silu": 0, "gelu_tanh": 1}  # the activations of a gated feed-forward's gate
+
+
+def _gate_act(act: str) -> int:
+    try:
+        return GATE_ACTS[act]
+    except KeyError:
+        raise KernelError(f"unknown gate activation {act!r} (known: {sorted(GATE_ACTS)})") from None
+
+
+def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, act: str = "silu") -> None:
+    """``out = act(gate) * up`` for rows ``[gate | up]``; ``act`` is ``silu`` or ``gelu_tanh``."""
     T, I2 = gate_up.shape
     if I2 % 2 or out.shape != (T, I2 // 2) or out.dtype != gate_up.dtype:
         raise KernelError("silu_mul: shapes or dtypes do not match")
-    _check(load().kvc_silu_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), T, I2 // 2,
-                               _code(out, "out"), _stream()), "kvc_silu_mul")
+    _check(load().kvc_gate_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), T, I2 // 2, _gate_act(act),
+                               _code(out, "out"), _stream()), "kvc_gate_mul")
 
 
 def gather_rows(out: torch.Tensor, src: torch.Tensor, rows: torch.Tensor) -> None:
@@ -354,11 +372,12 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
                     *, table: torch.Tensor, positions: torch.Tensor, token_req: torch.Tensor,
                     slots: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                     window: int = 0, dv: int | None = None, slopes: torch.Tensor | None = None,
-                    chunk: int = 0) -> None:
+                    chunk: int = 0, sinks: torch.Tensor | None = None) -> None:
     """``q`` is a ``[T, >= nh*d]`` view whose rows hold the query heads first.  ``dv``: the size
     of a value head where it differs from a key head's ``d`` (``out`` is ``[T, nh*dv]``).
     ``slopes`` (float32 ``[nh]``): ``slopes[h] * distance`` is taken off every score of head h;
-    ``chunk``: a token sees only the keys of its own chunk of that many positions."""
+    ``chunk``: a token sees only the keys of its own chunk of that many positions.  ``sinks``
+    (float32 ``[nh]``): ``exp(sinks[h])`` joins the softmax's denominator of head h."""
     if slopes is not None and (slopes.shape != (nh,) or slopes.dtype != torch.float32):
         raise KernelError("paged_attention: slopes must be float32 [nh]")
     T = out.shape[0]
@@ -377,7 +396,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         _dev(table, "table", torch.int32), table.shape[1],
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(slots, "slots", torch.int32), T, nh, nkv, d, dv, page_size, num_pages, float(scale),
-        int(window), None if slopes is None else _dev(slopes, "slopes"), int(chunk),
+        int(window), None if slopes is None else _dev(slopes, "slopes"), int(chunk), _sinks(sinks, nh),
         _code(out, "out"), _stream()), "kvc_paged_attention")
 
 
@@ -430,6 +449,15 @@ def _slopes(slopes: torch.Tensor | None, nh: int) -> int | None:
     if slopes.shape != (nh,):
         raise KernelError("attention: a distance slope per query head")
     return _dev(slopes, "slopes", torch.float32)
+
+
+def _sinks(sinks: torch.Tensor | None, nh: int) -> int | None:
+    """Pointer to the softmax sinks (float32, a value per query head) of the attention kernels."""
+    if sinks is None:
+        return None
+    if sinks.shape != (nh,):
+        raise KernelError("attention: a sink per query head")
+    return _dev(sinks, "sinks", torch.float32)
 
 
 def decode_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
@@ -516,7 +544,8 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
                      part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
                      sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False,
                      write_kv: bool = False, token_rows: torch.Tensor | None = None,
-                     slopes: torch.Tensor | None = None, chunk: int = 0) -> None:
+                     slopes: torch.Tensor | None = None, chunk: int = 0,
+                     sinks: torch.Tensor | None = None) -> None:
     """bfloat16 attention of single tokens on the matrix cores (see the C header), with the
     rotation of each token's query and key and the write of its key and value into the cache
     (``write_kv``) in the same kernel; ``qkv`` is not changed.  With ``rot_dim = 0`` and
@@ -555,7 +584,8 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
         None if token_rows is None else _dev(token_rows, "token_rows", torch.int32),
         c, s_, int(rot_dim), int(bool(interleaved)),
         int(bool(write_kv)), T, nh, nkv, d, page_size, num_pages, float(scale),
-        int(window), _slopes(slopes, nh), int(chunk), int(nsplit), _stream()), "kvc_decode_attention")
+        int(window), _slopes(slopes, nh), int(chunk), _sinks(sinks, nh), int(nsplit), _stream()),
+        "kvc_decode_attention")
 
 
 def prefill_attention_supported(nh: int, nkv: int, d: int, page_size: int, dtype: torch.dtype) -> bool:
@@ -568,7 +598,8 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       window: int = 0, nsplit: int = 1, part_o: torch.Tensor | None = None,
                       part_ml: torch.Tensor | None = None, cos: torch.Tensor | None = None,
                       sin: torch.Tensor | None = None, rot_dim: int = 0, interleaved: bool = False,
-                      slopes: torch.Tensor | None = None, chunk: int = 0) -> None:
+                      slopes: torch.Tensor | None = None, chunk: int = 0,
+                      sinks: torch.Tensor | None = None) -> None:
     """bfloat16 attention of portions of prompts on the matrix cores (see the C header).
     ``nsplit > 1`` deals every tile's keys to that many blocks; ``part_o`` (float32,
     ``T*nh*nsplit*d`` values) and ``part_ml`` (``T*nh*nsplit*2``) are then the workspace.
@@ -601,7 +632,7 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         _dev(table, "table", torch.int32), table.shape[1], _dev(positions, "positions", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs,
         nh, nkv, d, page_size, num_pages, float(scale), int(window), _slopes(slopes, nh), int(chunk),
-        po, pml, int(nsplit), cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved), _stream()),
+        _sinks(sinks, nh), po, pml, int(nsplit), cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved), _stream()),
         "kvc_prefill_attention")
 
 
@@ -797,8 +828,9 @@ def skinny_blocks(N: int, K: int, gated: bool = False, packed: bool = False) -> 
 
 
 def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: torch.Tensor,
-                  bias: torch.Tensor | None, gated: bool) -> ScaledRows | None:
-    """The weight-streaming product with a norm on either side folded in (see the C header)."""
+                  bias: torch.Tensor | None, gated: bool, act: str = "silu") -> ScaledRows | None:
+    """The weight-streaming product with a norm on either side folded in (see the C header);
+    ``act`` is the gate's activation of the gated form."""
     data = x.data if isinstance(x, ScaledRows) else x
     M, K = data.shape
     N = w.shape[0] // 2 if gated else w.shape[0]
@@ -842,7 +874,7 @@ def _fused_skinny(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows
         w_ptr, packed = _streamed(w, N)
         _check(load().kvc_gemm_skinny_fused_bf16(
             c_ptr, data.data_ptr(), w_ptr, None if bias is None else _dev(bias, "bias"), M, N, K,
-            data.stride(0), ldc, int(gated), in_ss or None, in_parts, in_width, float(in_eps),
+            data.stride(0), ldc, (1 + _gate_act(act)) if gated else 0, in_ss or None, in_parts, in_width, float(in_eps),
             residual, ldr, gain, out_ss, packed, _stream()), "kvc_gemm_skinny_fused_bf16")
     return result
 
@@ -880,9 +912,9 @@ def gemm_mid(out: torch.Tensor | None, x: torch.Tensor, w: torch.Tensor, bias: t
     """The weight-streaming product for up to 192 rows of bfloat16 whose waves share the rows
     through LDS, the faster one from 9 rows on (see the C header for the
     modes: 0 plain, 1 ``silu(gate) * up``, 2 partial sums of slices along K only, 3 plain
-    with slices and a kernel that sums them)."""
+    with slices and a kernel that sums them, 4 ``gelu_tanh(gate) * up``)."""
     M, K = x.shape
-    N = w.shape[0] // 2 if mode == 1 else w.shape[0]
+    N = w.shape[0] // 2 if mode in (1, 4) else w.shape[0]
     if w.shape[1] != K or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not x.is_cuda:
         raise KernelError("gemm_mid: operands must be bfloat16 GPU tensors with matching K")
     if not mid_operands_ok(x, w):
@@ -952,12 +984,13 @@ def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.
 
 
 def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Tensor,
-                    bias: torch.Tensor | None, scratch) -> None:
-    """``out = silu(x @ wg.T) * (x @ wu.T)`` with ``wg`` the first half of ``w``'s rows and
-    ``wu`` the second (biases likewise).  Few rows of bfloat16 run as one weight-streaming
-    kernel; otherwise ``scratch()`` gives the ``[M, 2I]`` buffer for the two-kernel form."""
+                    bias: torch.Tensor | None, scratch, act: str = "silu") -> None:
+    """``out = act(x @ wg.T) * (x @ wu.T)`` with ``wg`` the first half of ``w``'s rows and
+    ``wu`` the second (biases likewise); ``act`` is ``silu`` or ``gelu_tanh``.  Few rows of
+    bfloat16 run as one weight-streaming kernel; otherwise ``scratch()`` gives the ``[M, 2I]``
+    buffer for the two-kernel form."""
     if isinstance(x, ScaledRows):
-        _fused_skinny(out, x, w, bias, gated=True)
+        _fused_skinny(out, x, w, bias, gated=True, act=act)
         return
     M, K = x.shape
     I = w.shape[0] // 2
@@ -970,6 +1003,9 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             return
         if bias is not None and (bias.dtype != torch.bfloat16 or bias.shape != (2 * I,)):
             raise KernelError("linear_silu_mul: bias must be bfloat16 [2I]")
+        if act != "silu":
+            _fused_skinny(out, x, w, bias, gated=True, act=act)
+            return
         w_ptr, packed = _streamed(w, I)
         _check(load().kvc_gemm_skinny_silu_mul_bf16(
             out.data_ptr(), x.data_ptr(), w_ptr, None if bias is None else _dev(bias, "bias"),
@@ -979,11 +1015,11 @@ def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Te
             and x.is_cuda and mid_operands_ok(x, w) and out.stride(1) == 1
             and mid_rows_ok(M, bool(_streamed(w, I)[1]), MID_ROWS_GATED)):
         # 17 to 128 rows: the waves of a block share the rows through LDS
-        gemm_mid(out, x, w, bias, mode=1)
+        gemm_mid(out, x, w, bias, mode=4 if _gate_act(act) == 1 else 1)
         return
     gate_up = scratch()
     linear(gate_up, x, w, bias)
-    silu_mul(out, gate_up)
+    silu_mul(out, gate_up, act)
 
 
 def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: torch.Tensor,
@@ -1252,10 +1288,12 @@ def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
                       decay: torch.Tensor, beta: torch.Tensor | None, state: torch.Tensor, *,
                       positions: torch.Tensor, token_req: torch.Tensor, q_start: torch.Tensor,
                       slots: torch.Tensor, num_reqs: int, heads: int, qk_heads: int, dim: int,
-                      vdim: int, delta_rule: bool, q_scale: float = 1.0) -> None:
+                      vdim: int, delta_rule: bool = False, q_scale: float = 1.0,
+                      scalar_gates: bool = False) -> None:
     """The recurrence of a matrix state per head (see the C header): ``q, k [T, qk_heads * dim]``,
     ``v [T, heads * vdim]``, all float32 rows (column views are fine); ``decay [T, heads * dim]``
-    (a factor per key channel) or, with ``delta_rule``, ``decay`` and ``beta [T, heads]``;
+    (a factor per key channel) or, with ``delta_rule``, ``decay`` and ``beta [T, heads]``; with
+    ``scalar_gates`` the rule is ``S <- decay S + beta k v^T`` with the same two ``[T, heads]``;
     ``state [slots, heads, linear_state_rows(dim), vdim]`` float32, in an order of the kernel's own;
     ``out [T, heads * vdim]`` float32.  ``q_scale``
     multiplies every q on its way in."""
@@ -1271,17 +1309,21 @@ def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
     qp, qs = _f32_rows(q, "q", qk_heads * dim)
     kp, ks = _f32_rows(k, "k", qk_heads * dim)
     vp, vs = _f32_rows(v, "v", heads * vdim)
-    dp, ds = _f32_rows(decay, "decay", heads if delta_rule else heads * dim)
+    if delta_rule and scalar_gates:
+        raise KernelError("linear_state_scan: one rule at a time")
+    per_head = delta_rule or scalar_gates
+    dp, ds = _f32_rows(decay, "decay", heads if per_head else heads * dim)
     bp, bs = (0, 0)
-    if delta_rule:
+    if per_head:
         if beta is None or beta.shape[0] < T:
-            raise KernelError("linear_state_scan: the delta rule needs beta")
+            raise KernelError("linear_state_scan: this rule needs beta")
         bp, bs = _f32_rows(beta, "beta", heads)
     _check(load().kvc_linear_state_scan(
         out.data_ptr(), qp, qs, kp, ks, vp, vs, dp, ds, bp or None, bs, _dev(state, "state"),
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, heads,
-        qk_heads, dim, vdim, int(bool(delta_rule)), float(q_scale), _stream()), "kvc_linear_state_scan")
+        qk_heads, dim, vdim, 2 if scalar_gates else int(bool(delta_rule)), float(q_scale), _stream()),
+        "kvc_linear_state_scan")
 
 
 def sigmoid_power(out: torch.Tensor, z: torch.Tensor, bias: torch.Tensor | None, inv_tau: float) -> None:
@@ -1331,6 +1373,110 @@ def head_rmsnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, ga
     _check(load().kvc_head_rmsnorm_gate(_dev(out, "out"), _code(out, "out"), _dev(o, "o", torch.float32), gp, gs, gc,
                                         _dev(gain, "gain", torch.float32), float(eps), T, heads, vdim, _stream()),
            "kvc_head_rmsnorm_gate")
+
+
+def max_gates(keep: torch.Tensor, take: torch.Tensor, m_out: torch.Tensor, i_raw: torch.Tensor,
+              f_raw: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float,
+              m_state: torch.Tensor, *, positions: torch.Tensor, token_req: torch.Tensor,
+              q_start: torch.Tensor, slots: torch.Tensor, num_reqs: int) -> None:
+    """The gates of a matrix memory with log gates and a running maximum, per request in token
+    order (see the C header): ``keep, take, m_out [T, heads]`` float32 from the raw gate rows
+    ``i_raw, f_raw`` (float32, column views are fine); ``m_state [slots, heads]`` float32."""
+    T, nh = keep.shape
+    f = torch.float32
+    if take.shape != (T, nh) or m_out.shape != (T, nh) or i_bias.shape != (nh,) or f_bias.shape != (nh,) \
+            or m_state.dim() != 2 or m_state.shape[1] != nh or not m_state.is_contiguous() \
+            or i_raw.shape[0] < T or f_raw.shape[0] < T or q_start.numel() < num_reqs + 1:
+        raise KernelError("max_gates: shapes do not match")
+    for t in (keep, take, m_out):
+        if not t.is_contiguous():
+            raise KernelError("max_gates: the results must be contiguous")
+    ip, is_ = _f32_rows(i_raw, "i_raw", nh)
+    fp, fs = _f32_rows(f_raw, "f_raw", nh)
+    _check(load().kvc_max_gates(
+        _dev(keep, "keep", f), _dev(take, "take", f), _dev(m_out, "m_out", f), ip, is_, fp, fs,
+        _dev(i_bias, "i_bias", f), _dev(f_bias, "f_bias", f), float(cap), _dev(m_state, "m_state", f),
+        _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, nh, _stream()),
+        "kvc_max_gates")
+
+
+def max_gated_finish(out: torch.Tensor, o: torch.Tensor, m: torch.Tensor, gate: torch.Tensor,
+                     gain: torch.Tensor, eps: float, den_eps: float, heads: int, vdim: int) -> None:
+    """``y = o[..., :vdim] / (max(|o[..., vdim]|, exp(-m)) + den_eps)``; ``out = y / rms_head(y) *
+    gain * sigmoid(gate)``: ``o [T, heads * (vdim + 1)]`` float32 (the last column of a head is
+    the normaliser's product with the query), ``m [T, heads]``, ``gain [heads * vdim]``, the gate
+    rows of any dtype (a column view is fine)."""
+    T = o.shape[0]
+    if o.shape != (T, heads * (vdim + 1)) or out.shape != (T, heads * vdim) or not out.is_contiguous() \
+            or not o.is_contiguous() or gain.shape != (heads * vdim,) or m.shape != (T, heads) or not m.is_contiguous():
+        raise KernelError("max_gated_finish: shapes do not match")
+    gp, gs, gc = _rows(gate, "gate", heads * vdim)
+    _check(load().kvc_max_gated_finish(
+        _dev(out, "out"), _code(out, "out"), _dev(o, "o", torch.float32), _dev(m, "m", torch.float32), gp, gs, gc,
+        _dev(gain, "gain", torch.float32), float(eps), float(den_eps), T, heads, vdim, _stream()),
+        "kvc_max_gated_finish")
+
+
+def append_ones(out: torch.Tensor, v: torch.Tensor, heads: int, vdim: int) -> None:
+    """``out [T, heads * (vdim + 1)]`` float32: every head's ``vdim`` values of ``v`` (float32 rows, a
+    column view is fine) and a one behind them."""
+    T = out.shape[0]
+    if out.shape != (T, heads * (vdim + 1)) or not out.is_contiguous() or out.dtype != torch.float32 or v.shape[0] < T:
+        raise KernelError("append_ones: shapes do not match")
+    vp, vs = _f32_rows(v, "v", heads * vdim)
+    _check(load().kvc_append_ones(out.data_ptr(), vp, vs, T, heads, vdim, _stream()), "kvc_append_ones")
+
+
+def norm_add_norm(out: torch.Tensor | None, residual: torch.Tensor, delta: torch.Tensor,
+                  post_gain: torch.Tensor, eps: float, next_gain: torch.Tensor | None = None,
+                  next_eps: float | None = None) -> None:
+    """``residual += post_gain * delta / rms(delta)``, then, given ``out``, ``out = next_gain *
+    residual / rms(residual)``: the norm behind a sublayer, the sum into the float32 stream and the
+    norm before the next sublayer in one pass (both roots hold their eps).  ``delta`` is float32
+    or bfloat16."""
+    T, H = residual.shape
+    if delta.shape != (T, H) or not delta.is_contiguous() or not residual.is_contiguous() or post_gain.shape != (H,):
+        raise KernelError("norm_add_norm: shapes do not match")
+    if out is not None and (out.shape != (T, H) or not out.is_contiguous() or next_gain is None
+                            or next_gain.shape != (H,)):
+        raise KernelError("norm_add_norm: the second norm's rows or gain do not fit")
+    _check(load().kvc_norm_add_norm(
+        None if out is None else _dev(out, "out"), 0 if out is None else _code(out, "out"),
+        _dev(residual, "residual", torch.float32), _dev(delta, "delta"), _code(delta, "delta"),
+        _dev(post_gain, "post_gain", torch.float32), float(eps),
+        None if out is None else _dev(next_gain, "next_gain", torch.float32),
+        float(eps if next_eps is None else next_eps), T, H, _stream()), "kvc_norm_add_norm")
+
+
+def wide_qk_norm(qkv: torch.Tensor, q_gain: torch.Tensor, k_gain: torch.Tensor, eps: float, *,
+                 copy_k: bool = False) -> None:
+    """Rows of ``qkv`` start with all query heads (as many values as ``q_gain`` has) and all key
+    heads (``k_gain``): each of the two runs is divided by its root mean square as a whole and
+    multiplied by its gain, in place.  With ``copy_k`` the keys as they were are first copied
+    behind themselves (where a layer's values are its keys as projected)."""
+    nq, nk = q_gain.numel(), k_gain.numel()
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < nq + nk * (2 if copy_k else 1):
+        raise KernelError("wide_qk_norm: rows too short")
+    _check(load().kvc_wide_qk_norm(qkv.data_ptr(), qkv.stride(0), _dev(q_gain, "q_gain", torch.float32),
+                                   _dev(k_gain, "k_gain", torch.float32), float(eps), qkv.shape[0], nq, nk,
+                                   int(bool(copy_k)), _code(qkv, "qkv"), _stream()), "kvc_wide_qk_norm")
+
+
+def head_gate(out: torch.Tensor, x: torch.Tensor, gate: torch.Tensor, *, heads: int, head_stride: int,
+              skip: int, n: int) -> None:
+    """``out[t, h, :n] = x[t, h, skip : skip + n] * sigmoid(gate[t, h])``: ``x`` rows of ``heads`` heads of
+    ``head_stride`` values, ``gate`` rows of ``heads`` values (column views are fine),
+    ``out [T, heads * n]``, all of one dtype."""
+    T = out.shape[0]
+    if out.shape != (T, heads * n) or not out.is_contiguous() or out.dtype != x.dtype or x.stride(1) != 1 \
+            or x.shape[0] < T or x.shape[1] < heads * head_stride or gate.shape[0] < T:
+        raise KernelError("head_gate: shapes do not match")
+    gp, gs, gc = _rows(gate, "gate", heads)
+    if gc != _code(x, "x"):
+        raise KernelError("head_gate: the gate has another dtype than the rows")
+    _check(load().kvc_head_gate(out.data_ptr(), x.data_ptr(), x.stride(0), gp, gs, T, heads, head_stride, skip, n,
+                                _code(out, "out"), _stream()), "kvc_head_gate")
 
 
 def moe_route(choice: torch.Tensor, weight: torch.Tensor, logits: torch.Tensor, *, top: int, groups: int = 1,

@@ -1,6 +1,7 @@
 """Parts: importing the package registers the built-in kinds."""
 
-from . import (attention, block, embedding, layernorm, linear_attention, mlp, moe, parallel, recurrent,  # noqa: F401
+from . import (attention, block, embedding, latent_attention, layernorm, linear_attention, mlp, moe, parallel,  # noqa: F401
+               recurrent,
                rmsnorm, rotary, stream)  # noqa: F401
 from .base import (  # noqa: F401
     BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, Block, CacheNeed,

@@ -94,6 +94,8 @@ class PagedAttention(Mixer):
     llama3.py:60); ``window`` 0 attends to every earlier token; ``page_size`` asks for cache
     pages of that many tokens for this layer's group (None: the engine's block size)."""
 
+    any_head_size = False  # a subclass whose heads need not be a multiple of 16 takes the general kernels then
+
     @property
     def takes_scaled_rows(self) -> bool:  # x only goes into the qkv product
         return self.hidden_size % 8 == 0
@@ -107,7 +109,8 @@ class PagedAttention(Mixer):
                  v_head_dim: int | None = None, qk_norm_eps: float | None = None,
                  tensor_names: dict[str, str] | None = None, float32_result: bool = False,
                  qk_norm_gain: bool = True, distance_slopes: tuple[float, ...] | None = None,
-                 chunk: int = 0, position: PositionEncoding | None = None) -> None:
+                 chunk: int = 0, qk_norm_span: str = "head", values_are_keys: bool = False,
+                 sinks: bool = False, position: PositionEncoding | None = None) -> None:
         """``v_head_dim``: the size of a value head where it differs from ``head_dim``, the
         size of a query and key head.  ``qk_norm_eps`` (None: no such norm): every query and
         key head is divided by its root mean square, eps inside the root, and multiplied by a
@@ -118,13 +121,28 @@ class PagedAttention(Mixer):
         the heads has no gain (and no tensors).  ``distance_slopes``: a value per query head;
         ``slope * (i - j)`` is taken off the score of query i and key j before the softmax (no
         rotation is needed for such a layer).  ``chunk`` > 0: query i sees key j <= i only if
-        both lie in the same chunk of that many positions, counted from the sequence's start."""
+        both lie in the same chunk of that many positions, counted from the sequence's start.
+        ``qk_norm_span`` ``"projection"``: the norm spans all query heads at once (and all key
+        heads at once), with a gain of that whole size each, instead of every head alone.
+        ``values_are_keys``: there is no value projection; a token's values are its keys as
+        projected, before norm and rotation.  ``sinks``: a learned score per query head (tensor
+        ``sink``) that joins the softmax's denominator without a key or a value, unscaled."""
+        if qk_norm_span not in ("head", "projection"):
+            raise ValueError(f"qk_norm_span is 'head' or 'projection', got {qk_norm_span!r}")
+        if qk_norm_span == "projection" and (qk_norm_eps is None or not qk_norm_gain):
+            raise ValueError("a norm over the whole projection needs its eps and has gains")
+        if values_are_keys and v_head_dim not in (None, head_dim):
+            raise ValueError("values that are the keys have the keys' size")
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         v_head_dim = head_dim if v_head_dim is None else v_head_dim
-        plain = v_head_dim == head_dim and qk_norm_eps is None
+        self.head_norm = qk_norm_eps is not None and qk_norm_span == "head"
+        self.wide_norm = qk_norm_eps is not None and qk_norm_span == "projection"
+        plain = v_head_dim == head_dim and not self.head_norm
         if plain and (head_dim % 16 or head_dim > 256):
-            raise ValueError(f"head size {head_dim} is not supported (multiples of 16 up to 256)")
+            if qk_norm_eps is None and not values_are_keys and not self.any_head_size:
+                raise ValueError(f"head size {head_dim} is not supported (multiples of 16 up to 256)")
+            plain = False  # the kernel that rotates and writes heads of any size, and the general attention
         if not 0 < head_dim <= 256 or not 0 < v_head_dim <= 256:
             raise ValueError(f"head sizes {head_dim} and {v_head_dim} are not supported (1 to 256)")
         self.hidden_size = hidden_size
@@ -134,6 +152,8 @@ class PagedAttention(Mixer):
         self.v_head_dim = v_head_dim
         self.qk_norm_eps = qk_norm_eps
         self.qk_norm_gain = bool(qk_norm_gain)
+        self.values_are_keys = bool(values_are_keys)
+        self.has_sinks = bool(sinks)
         if distance_slopes is not None and len(distance_slopes) != num_heads:
             raise ValueError(f"{len(distance_slopes)} distance slopes for {num_heads} heads")
         if chunk < 0:
@@ -159,18 +179,20 @@ class PagedAttention(Mixer):
         self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight",
                       "o": "o_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
                       "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-                      "o_bias": "o_proj.bias", **(tensor_names or {})}
+                      "o_bias": "o_proj.bias", "sink": "sinks", **(tensor_names or {})}
 
     def param_specs(self) -> list[ParamSpec]:
         total = self.q_size + self.kv_size + self.v_size
         n = self.names
 
+        if self.values_are_keys:  # no value projection: q and k alone
+            total = self.q_size + self.kv_size
+
         def stacked(q: str, k: str, v: str) -> tuple[ParamSource, ...]:
-            return (
-                ParamSource(n[q], 0, self.q_size),
-                ParamSource(n[k], self.q_size, self.kv_size),
-                ParamSource(n[v], self.q_size + self.kv_size, self.v_size),
-            )
+            qk = (ParamSource(n[q], 0, self.q_size), ParamSource(n[k], self.q_size, self.kv_size))
+            if self.values_are_keys:
+                return qk
+            return (*qk, ParamSource(n[v], self.q_size + self.kv_size, self.v_size))
 
         specs = [
             ParamSpec("qkv_proj.weight", (total, self.hidden_size), sources=stacked("q", "k", "v")),
@@ -183,9 +205,13 @@ class PagedAttention(Mixer):
             specs.append(ParamSpec("o_proj.bias", (self.hidden_size,), init="zeros",
                                    sources=(ParamSource(n["o_bias"], 0, self.hidden_size),)))
         if self.qk_norm_eps is not None and self.qk_norm_gain:
-            for key in ("q_norm", "k_norm"):
-                specs.append(ParamSpec(key, (self.head_dim,), kind="vector", init="gain",
-                                       sources=(ParamSource(n[key], 0, self.head_dim),)))
+            for key, whole in (("q_norm", self.q_size), ("k_norm", self.kv_size)):
+                size = whole if self.wide_norm else self.head_dim
+                specs.append(ParamSpec(key, (size,), kind="vector", init="gain",
+                                       sources=(ParamSource(n[key], 0, size),)))
+        if self.has_sinks:
+            specs.append(ParamSpec("sinks", (self.num_heads,), kind="vector", init="normal",
+                                   sources=(ParamSource(n["sink"], 0, self.num_heads),)))
         return specs
 
     def setup(self, runtime) -> None:
@@ -193,7 +219,7 @@ class PagedAttention(Mixer):
         self._slopes = self._unit_gain = None
         if self.distance_slopes is not None:
             self._slopes = torch.tensor(self.distance_slopes, dtype=torch.float32, device=runtime.device)
-        if self.qk_norm_eps is not None and not self.qk_norm_gain:
+        if self.head_norm and not self.qk_norm_gain:
             self._unit_gain = torch.ones(self.head_dim, dtype=torch.float32, device=runtime.device)
 
     def cache_need(self) -> CacheNeed:
@@ -229,12 +255,31 @@ class PagedAttention(Mixer):
         return self.v_plane_dim == self.head_dim
 
     def forward(self, x, ctx, call, sink=None):
+        return self._output(self._attention(self._project(x, ctx), ctx, call), ctx, sink)
+
+    def _project(self, x, ctx):
+        """Rows ``[q heads | k heads | v heads]`` for the step's tokens, normed over the whole
+        projection where the layer says so (norms of single heads and rotation come later)."""
         p = self.params
         # step buffers are named by their width: layers of one model may differ in size
         qkv = ctx.buf(_sized("attn_qkv", self.q_size + self.kv_size + self.v_size, self.plain),
                       self.q_size + self.kv_size + self.v_size)
-        ops.linear(qkv, x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
+        if self.values_are_keys:
+            ops.linear(qkv[:, : self.q_size + self.kv_size], x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
+            if not self.wide_norm:  # the values are the keys as projected
+                qkv[:, self.q_size + self.kv_size:].copy_(qkv[:, self.q_size: self.q_size + self.kv_size])
+        else:
+            ops.linear(qkv, x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
+        if self.wide_norm:
+            # one norm over all query heads and one over all key heads, each with a gain of its
+            # whole size; the raw keys become the values on the way where the layer says so
+            ops.wide_qk_norm(qkv, p["q_norm"], p["k_norm"], self.qk_norm_eps, copy_k=self.values_are_keys)
+        return qkv
 
+    def _attention(self, qkv, ctx, call):
+        """Norm of the heads, rotation, the cache write and the attention itself for rows ``qkv``;
+        returns ``[T, heads * value size]`` in a step buffer."""
+        p = self.params
         group = ctx.groups[call.group_index]
         # K pages [kv_heads, page, d]; V pages [kv_heads, dv, page]: the keys of a page lie
         # side by side, which is how the matrix cores want the values.  Values wider than the
@@ -257,7 +302,8 @@ class PagedAttention(Mixer):
             ops.qk_norm_rope_kv_write(qkv, k_cache, v_planes, cos, sin, rot_dim=rot_dim,
                                       interleaved=interleaved, kv_slot=kv_slot, nh=self.num_heads,
                                       nkv=self.num_kv_heads, d=self.head_dim, dv=self.v_head_dim,
-                                      q_gain=p.get("q_norm", self._unit_gain), k_gain=p.get("k_norm", self._unit_gain),
+                                      q_gain=p.get("q_norm", self._unit_gain) if self.head_norm else None,
+                                      k_gain=p.get("k_norm", self._unit_gain) if self.head_norm else None,
                                       eps=self.qk_norm_eps or 0.0, write_kv=call.write_cache)
             rot_dim, interleaved = 0, False
             cos = sin = ctx.buffers.get("rope_none", ctx.num_tokens, 0, torch.float32)
@@ -274,6 +320,10 @@ class PagedAttention(Mixer):
                              rot_dim, interleaved, prepared)
             attn.view(T, self.num_heads, m, self.v_plane_dim).copy_(
                 parts.view(m, T, self.num_heads, self.v_plane_dim).permute(1, 2, 0, 3))
+        return attn
+
+    def _output(self, attn, ctx, sink=None):
+        p = self.params
         if sink is not None:
             return ops.linear(sink, attn, p["o_proj.weight"], p.get("o_proj.bias"))
         if self.float32_result:
@@ -292,7 +342,7 @@ class PagedAttention(Mixer):
                       scale=self.scale, window=self.window)
         x_dtype = qkv.dtype
         # a distance bias and a chunked view are options of every attention kernel
-        common.update(slopes=self._slopes, chunk=self.chunk)
+        common.update(slopes=self._slopes, chunk=self.chunk, sinks=self.params.get("sinks"))
         # a token never sees more keys than its window or its chunk holds: what the launch plans count
         reach = min((n for n in (self.window, self.chunk) if n > 0), default=0)
         if not self._same_sizes():
@@ -349,7 +399,7 @@ class PagedAttention(Mixer):
                                       positions=ctx.positions, q_start=ctx.q_start, slots=ctx.slots,
                                       num_reqs=ctx.num_reqs, nh=self.num_heads, nkv=self.num_kv_heads,
                                       d=self.head_dim, scale=self.scale, window=self.window,
-                                      slopes=self._slopes, chunk=self.chunk,
+                                      slopes=self._slopes, chunk=self.chunk, sinks=self.params.get("sinks"),
                                       nsplit=nsplit, part_o=part_o, part_ml=part_ml,
                                       **(dict(cos=cos, sin=sin, rot_dim=rot_dim, interleaved=interleaved)
                                          if rotates else {}))

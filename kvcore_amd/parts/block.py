@@ -139,5 +139,74 @@ class ParallelResidualBlock(Block):
         return None
 
 
+class SandwichNormBlock(Block):
+    """A norm before and a norm behind each sublayer: ``r += post_mixer(mixer(pre_mixer(r)));
+    r += post_ffn(ffn(pre_ffn(r)))``, all four RMS norms with a gain.  Between two sublayers the
+    norm of the result, the sum into the float32 stream and the next sublayer's first norm are one
+    kernel (``ops.norm_add_norm``); so the block hands the next block its first norm's rows where
+    that block says it takes them (``input_gain``), and takes its own from the block before.  With
+    a feed-forward of kind ``none`` the layer is its first half."""
+
+    def __init__(self, *, mixer: Mixer, ffn: FeedForward, norms: dict[str, Norm],
+                 mixer_name: str = "mixer", ffn_name: str = "mlp", pre_mixer: str = "norm1",
+                 post_mixer: str = "norm1b", pre_ffn: str = "norm2", post_ffn: str = "norm2b") -> None:
+        super().__init__(mixer=mixer, ffn=ffn, norms=norms)
+        self.mixer_only = bool(getattr(ffn, "absent", False))
+        self.mixer_name, self.ffn_name = mixer_name, ffn_name
+        self.norm_names = (pre_mixer, post_mixer) if self.mixer_only else (pre_mixer, post_mixer, pre_ffn, post_ffn)
+        missing = [n for n in self.norm_names if n not in norms]
+        if missing or len(set(self.norm_names)) != len(self.norm_names):
+            raise ValueError(f"a block with norms on both sides of its sublayers needs {self.norm_names}; "
+                             f"given {list(norms)}")
+
+    def children(self) -> dict[str, Part]:
+        out: dict[str, Part] = {n: self.norms[n] for n in self.norm_names}
+        out[self.mixer_name] = self.mixer
+        if not self.mixer_only:
+            out[self.ffn_name] = self.ffn
+        return out
+
+    def input_gain(self, scaled: bool = True):
+        # finished rows are welcome; rows whose norm the mixer's first product would have to
+        # finish are not (the mixers of such layers read their input more than once)
+        return None if scaled else self.norms[self.norm_names[0]].as_gain()
+
+    def _gain(self, i: int):
+        gain = self.norms[self.norm_names[i]].as_gain()
+        if gain is None:
+            raise RuntimeError(f"norm {self.norm_names[i]!r} is not an RMS norm with a gain")
+        return gain
+
+    def _join(self, result, residual, ctx, post, following, name: str):
+        """``residual += post(result)``, and the rows of the norm ``following`` (a (gain, eps) or
+        None) into the step buffer ``name``."""
+        post_gain, post_eps = post
+        if following is None:
+            ops.norm_add_norm(None, residual, result, post_gain, post_eps)
+            return None
+        rows = ctx.buf(name, residual.shape[1])
+        ops.norm_add_norm(rows, residual, result, post_gain, post_eps, following[0], following[1])
+        return rows
+
+    def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
+        if isinstance(delta, ops.ScaledRows):
+            raise RuntimeError("this block takes finished rows or the stream, not rows still to be scaled")
+        if isinstance(delta, ops.NormedRows):
+            x = delta.data  # the block before made this block's first norm
+        else:
+            x = ctx.buf("block_x", residual.shape[1])
+            self.norms[self.norm_names[0]].forward_fused(x, residual, delta)
+        following = next_block.input_gain(scaled=False) if next_block is not None else None
+        a = self.mixer.forward(x, ctx, call)
+        if self.mixer_only:
+            rows = self._join(a, residual, ctx, self._gain(1), following, "block_x")
+            return None if rows is None else ops.NormedRows(rows)
+        x2 = self._join(a, residual, ctx, self._gain(1), self._gain(2), "block_x2")
+        f = self.ffn.forward(x2, ctx, call)
+        rows = self._join(f, residual, ctx, self._gain(3), following, "block_x")
+        return None if rows is None else ops.NormedRows(rows)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("sandwich_norm", SandwichNormBlock)
 register_block("parallel_residual", ParallelResidualBlock)

@@ -192,5 +192,84 @@ class GatedDeltaRule(_MatrixStateMixer):
         return self._finish(o, proj[:, self.conv_dim: self.conv_dim + inner], ctx)
 
 
+class MaxGatedMatrixMemory(_MatrixStateMixer):
+    """The matrix memory of the xLSTM family (mLSTM): per head ``S [dim, vdim]``, a normaliser ``n
+    [dim]`` and a running maximum ``m`` of the log gates, which starts at 0:
+
+        i = cap tanh((W_i h + b_i) / cap),   f = logsigmoid(cap tanh((W_f h + b_f) / cap))
+        m_t = max(f + m_(t-1), i)
+        S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T      (n likewise with k alone)
+        o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + den_eps),           q = W_q h * q_scale.
+
+    The normaliser is one more column of the state (the values get a column of ones), so the
+    recurrence is the scan of the other matrix-state mixers with two scalar gates a head.  Then
+    each head's ``o`` over its root mean square, times a gain of all heads' size, times
+    ``sigmoid(W_g h)``, and the output product.  ``tensor_names`` renames checkpoint tensors
+    (keys: q, k, v, g, o, norm, i, f, i_bias, f_bias)."""
+
+    def __init__(self, *, hidden_size: int, heads: int, dim: int, vdim: int, gate_cap: float, eps: float,
+                 den_eps: float = 1e-6, q_scale: float | None = None, tensor_names: dict[str, str] | None = None,
+                 float32_result: bool = False, position=None) -> None:
+        if min(heads, dim, vdim) <= 0 or not gate_cap > 0:
+            raise ValueError("a matrix memory needs positive sizes and a positive gate cap")
+        self.hidden_size, self.heads, self.dim, self.vdim = hidden_size, heads, dim, vdim
+        self.cap, self.eps, self.den_eps = float(gate_cap), eps, float(den_eps)
+        self.q_scale = dim ** -0.5 if q_scale is None else float(q_scale)
+        self.float32_result = float32_result
+        self.qk, self.inner = heads * dim, heads * vdim
+        self.names = {"q": "q.weight", "k": "k.weight", "v": "v.weight", "g": "g.weight", "o": "o.weight",
+                      "norm": "norm.weight", "i": "i.weight", "f": "f.weight", "i_bias": "i.bias", "f_bias": "f.bias",
+                      **(tensor_names or {})}
+
+    def param_specs(self) -> list[ParamSpec]:
+        n, H, nh = self.names, self.hidden_size, self.heads
+        return [
+            ParamSpec("in_proj.weight", (2 * self.qk + 2 * self.inner + 2 * nh, H), sources=_stacked(
+                [(n["q"], self.qk), (n["k"], self.qk), (n["v"], self.inner), (n["g"], self.inner),
+                 (n["i"], nh), (n["f"], nh)])),
+            ParamSpec("i.bias", (nh,), kind="vector", init="normal", sources=_src(n["i_bias"], nh)),
+            ParamSpec("f.bias", (nh,), kind="vector", init="normal", sources=_src(n["f_bias"], nh)),
+            ParamSpec("norm", (self.inner,), kind="vector", init="gain", sources=_src(n["norm"], self.inner)),
+            ParamSpec("o.weight", (H, self.inner), sources=_src(n["o"], H)),
+        ]
+
+    def product_weights(self) -> tuple[str, ...]:
+        return ("in_proj.weight", "o.weight")
+
+    def state_needs(self) -> tuple[StateNeed, ...]:
+        # the matrices with the normaliser as their last column, and the running maxima
+        return (StateNeed((self.heads, ops.linear_state_rows(self.dim), self.vdim + 1)), StateNeed((self.heads,)))
+
+    def forward(self, x, ctx, call, sink=None):
+        p, qk, inner, nh = self.params, self.qk, self.inner, self.heads
+        state, maxima = (ctx.states[i] for i in call.state_indices)
+        batch = self._batch(ctx)
+        width = 2 * qk + 2 * inner + 2 * nh
+        proj = ctx.buf(f"mm_proj:{width}", width, torch.float32)
+        ops.linear(proj, x, p["in_proj.weight"])
+        keep = ctx.buf(f"mm_keep:{nh}", nh, torch.float32)
+        take = ctx.buf(f"mm_take:{nh}", nh, torch.float32)
+        m = ctx.buf(f"mm_max:{nh}", nh, torch.float32)
+        at = 2 * qk + 2 * inner
+        ops.max_gates(keep, take, m, proj[:, at:at + nh], proj[:, at + nh:], p["i.bias"], p["f.bias"], self.cap,
+                      maxima, **batch)
+        wide = nh * (self.vdim + 1)
+        v1 = ctx.buf(f"mm_v:{wide}", wide, torch.float32)
+        ops.append_ones(v1, proj[:, 2 * qk:2 * qk + inner], nh, self.vdim)
+        o = ctx.buf(f"mm_o:{wide}", wide, torch.float32)
+        ops.linear_state_scan(o, proj[:, :qk], proj[:, qk:2 * qk], v1, keep, take, state, heads=nh, qk_heads=nh,
+                              dim=self.dim, vdim=self.vdim + 1, scalar_gates=True, q_scale=self.q_scale, **batch)
+        normed = ctx.buf(f"ms_normed:{inner}", inner)
+        ops.max_gated_finish(normed, o, m, proj[:, 2 * qk + inner:2 * qk + 2 * inner], p["norm"], self.eps,
+                             self.den_eps, nh, self.vdim)
+        if self.float32_result:
+            out = ctx.buf("mixer_out_f32", self.hidden_size, torch.float32)
+        else:
+            out = ctx.buf("mixer_out", self.hidden_size)
+        ops.linear(out, normed, p["o.weight"])
+        return out
+
+
 register_mixer("gated_linear_attention", GatedLinearAttention)
+register_mixer("max_gated_matrix_memory", MaxGatedMatrixMemory)
 register_mixer("gated_delta_rule", GatedDeltaRule)

@@ -1,4 +1,5 @@
-"""Gated feed-forward: ``down(silu(gate(x)) * up(x))`` with gate and up stacked.
+"""Gated feed-forward: ``down(act(gate(x)) * up(x))`` with gate and up stacked; ``act`` is silu
+unless the layer names another (``gelu_tanh``).
 
 Reference: kvcore/model/models/llama3.py:25-45 (gate rows first, then up rows) and
 kvcore/model/layer/activation.py:14-16.
@@ -20,16 +21,22 @@ class SwiGLU(FeedForward):
 
     @property
     def takes_sink(self) -> bool:
-        return self.intermediate_size % 8 == 0
+        return self.intermediate_size % 8 == 0 and not self.float32_result
 
     def __init__(self, *, hidden_size: int, intermediate_size: int, bias: bool = False,
                  gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj",
-                 suffix: str = ".weight", sized_buffers: bool = False) -> None:
+                 suffix: str = ".weight", sized_buffers: bool = False, activation: str = "silu",
+                 float32_result: bool = False) -> None:
         """``gate_name``, ``up_name`` and ``down_name`` are the checkpoint's names of the three
         matrices relative to the part's prefix, ``suffix`` what follows each (biases end in
         ``.bias``).  ``sized_buffers``: name the step buffers by their width, for a model whose
         layers may differ in width (a buffer whose width changed from layer to layer would be
-        allocated anew at every layer)."""
+        allocated anew at every layer).  ``activation``: the gate's, ``silu`` or ``gelu_tanh``.
+        ``float32_result``: the output rows are float32 sums, for a consumer that normalises them."""
+        if activation not in ops.GATE_ACTS:
+            raise ValueError(f"gate activation {activation!r} is not supported (supported: {sorted(ops.GATE_ACTS)})")
+        self.activation = activation
+        self.float32_result = float32_result
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.bias = bias
@@ -66,10 +73,14 @@ class SwiGLU(FeedForward):
         act = ctx.buf(self._buf("ffn_act"), self.intermediate_size)
         # few rows: the product and the activation are one kernel and gate_up is never stored
         ops.linear_silu_mul(act, x, p["gate_up_proj.weight"], p.get("gate_up_proj.bias"),
-                            lambda: ctx.buf(self._buf("ffn_gate_up"), 2 * self.intermediate_size))
+                            lambda: ctx.buf(self._buf("ffn_gate_up"), 2 * self.intermediate_size),
+                            act=self.activation)
         if sink is not None:
             return ops.linear(sink, act, p["down_proj.weight"], p.get("down_proj.bias"))
-        out = ctx.buf("ffn_out", self.hidden_size)
+        if self.float32_result:
+            out = ctx.buf("ffn_out_f32", self.hidden_size, torch.float32)
+        else:
+            out = ctx.buf("ffn_out", self.hidden_size)
         ops.linear(out, act, p["down_proj.weight"], p.get("down_proj.bias"))
         return out
 

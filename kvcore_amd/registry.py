@@ -72,5 +72,10 @@ def _register_builtin() -> None:
     register_architecture("Vovalix", VovalixConfig.from_dict, vovalix_spec,
                           complete_config=complete_from_tensor_shapes)
 
+    from kvcore_amd.config.tazunex_config import TazunexConfig
+    from kvcore_amd.models.tazunex import tazunex_spec
+
+    register_architecture("Tazunex", TazunexConfig.from_dict, tazunex_spec)
+
 
 _register_builtin()
