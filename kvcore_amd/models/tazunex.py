@@ -63,7 +63,7 @@ def tazunex_spec(config: TazunexConfig) -> ModelSpec:
             mixer = PartSpec("paged_attention", {
                 "hidden_size": H, "num_heads": m.heads, "num_kv_heads": m.kv_heads, "head_dim": m.dim,
                 "scale": m.scale, "window": m.window, "qk_norm_eps": eps, "qk_norm_span": "projection",
-                "values_are_keys": True, "sinks": True, "float32_result": True,
+                "values_are_keys": True, "sinks": True, "float32_result": True, "sized_buffers": True,
                 "tensor_names": {"q": "q", "k": "k", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm",
                                  "sink": "sink"}})
         elif isinstance(m, LatentAttentionConfig):

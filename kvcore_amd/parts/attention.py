@@ -110,7 +110,8 @@ class PagedAttention(Mixer):
                  tensor_names: dict[str, str] | None = None, float32_result: bool = False,
                  qk_norm_gain: bool = True, distance_slopes: tuple[float, ...] | None = None,
                  chunk: int = 0, qk_norm_span: str = "head", values_are_keys: bool = False,
-                 sinks: bool = False, position: PositionEncoding | None = None) -> None:
+                 sinks: bool = False, sized_buffers: bool = False,
+                 position: PositionEncoding | None = None) -> None:
         """``v_head_dim``: the size of a value head where it differs from ``head_dim``, the
         size of a query and key head.  ``qk_norm_eps`` (None: no such norm): every query and
         key head is divided by its root mean square, eps inside the root, and multiplied by a
@@ -126,7 +127,9 @@ class PagedAttention(Mixer):
         heads at once), with a gain of that whole size each, instead of every head alone.
         ``values_are_keys``: there is no value projection; a token's values are its keys as
         projected, before norm and rotation.  ``sinks``: a learned score per query head (tensor
-        ``sink``) that joins the softmax's denominator without a key or a value, unscaled."""
+        ``sink``) that joins the softmax's denominator without a key or a value, unscaled.
+        ``sized_buffers``: name the step buffers by their width, for a model whose attention layers
+        differ in size."""
         if qk_norm_span not in ("head", "projection"):
             raise ValueError(f"qk_norm_span is 'head' or 'projection', got {qk_norm_span!r}")
         if qk_norm_span == "projection" and (qk_norm_eps is None or not qk_norm_gain):
@@ -171,6 +174,8 @@ class PagedAttention(Mixer):
         self.v_size = num_kv_heads * v_head_dim
         self.o_size = num_heads * v_head_dim
         self.plain = plain
+        # layers that are all alike share one step buffer a role; others name theirs by width
+        self.shared_buffers = plain and not sized_buffers and not self.any_head_size
         # values wider than the keys by a whole factor (up to four) are kept in that many cache
         # planes of the keys' size, so that the kernels for keys and values of one size serve them
         factor = v_head_dim // head_dim if v_head_dim % head_dim == 0 else 0
@@ -262,7 +267,7 @@ class PagedAttention(Mixer):
         projection where the layer says so (norms of single heads and rotation come later)."""
         p = self.params
         # step buffers are named by their width: layers of one model may differ in size
-        qkv = ctx.buf(_sized("attn_qkv", self.q_size + self.kv_size + self.v_size, self.plain),
+        qkv = ctx.buf(_sized("attn_qkv", self.q_size + self.kv_size + self.v_size, self.shared_buffers),
                       self.q_size + self.kv_size + self.v_size)
         if self.values_are_keys:
             ops.linear(qkv[:, : self.q_size + self.kv_size], x, p["qkv_proj.weight"], p.get("qkv_proj.bias"))
@@ -293,7 +298,7 @@ class PagedAttention(Mixer):
             rot_dim, interleaved = 0, False
         else:
             cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
-        attn = ctx.buf(_sized("attn_out", self.o_size, self.plain), self.o_size)
+        attn = ctx.buf(_sized("attn_out", self.o_size, self.shared_buffers), self.o_size)
         # with a norm of the heads, or values of another size than the keys, one kernel norms,
         # rotates and writes the cache; the attention kernels then take q and the cache as they are
         prepared = not self.plain
@@ -360,7 +365,7 @@ class PagedAttention(Mixer):
                 # for the largest at once, since a buffer that grows drops the graphs
                 most = (decode_target_blocks() // self.num_kv_heads + 1 + max(T, ctx.buffers.seq_capacity)) \
                     * self.num_heads
-                part_o = ctx.buffers.get(_sized("attn_part_o", self.head_dim, self.plain),
+                part_o = ctx.buffers.get(_sized("attn_part_o", self.head_dim, self.shared_buffers),
                                          T * self.num_heads * nsplit, self.head_dim,
                                          torch.float32, reserve=most)
                 part_ml = ctx.buffers.get("attn_part_ml", T * self.num_heads * nsplit, 2, torch.float32,
@@ -390,7 +395,7 @@ class PagedAttention(Mixer):
                 if nsplit > 1:
                     # asked for at their largest at once: a buffer that grows drops the graphs
                     most = prefill_split_rows(self.num_kv_heads, self.num_heads // self.num_kv_heads) * self.num_heads
-                    part_o = ctx.buffers.get(_sized("attn_prefill_part_o", self.head_dim, self.plain),
+                    part_o = ctx.buffers.get(_sized("attn_prefill_part_o", self.head_dim, self.shared_buffers),
                                              T * self.num_heads * nsplit,
                                              self.head_dim, torch.float32, reserve=most)
                     part_ml = ctx.buffers.get("attn_prefill_part_ml", T * self.num_heads * nsplit, 2,
