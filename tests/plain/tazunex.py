@@ -40,10 +40,16 @@ def rotate(x: torch.Tensor, positions: torch.Tensor, dims: int, base: float, int
     return out
 
 
-def window_softmax(scores: torch.Tensor, window: int, sink: torch.Tensor | None) -> torch.Tensor:
+def window_of(m: dict) -> int | None:
+    """The mixer's window, None where its configuration names none (every earlier token is seen)."""
+    return (m.get("mask") or {}).get("size")
+
+
+def window_softmax(scores: torch.Tensor, window: int | None, sink: torch.Tensor | None) -> torch.Tensor:
     """``scores [heads, T, T]`` -> weights; query i sees key j with ``0 <= i - j < window``; with
     ``sink [heads]`` the denominator also holds ``exp(sink)``."""
     T = scores.shape[-1]
+    window = T + 1 if window is None else window
     i = torch.arange(T)[:, None]
     j = torch.arange(T)[None, :]
     seen = (j <= i) & (i - j < window)
@@ -69,13 +75,14 @@ def sink_attention(h: torch.Tensor, w: dict, m: dict, eps: float) -> torch.Tenso
     q = (rms(q, eps) * w["q.norm"]).view(T, H, d)
     kk = (rms(k, eps) * w["k.norm"]).view(T, G, d)
     pos = torch.arange(T)
-    q = rotate(q, pos, m["rot"]["dims"], m["rot"]["base"], False)
-    kk = rotate(kk, pos, m["rot"]["dims"], m["rot"]["base"], False)
+    if m.get("rot"):
+        q = rotate(q, pos, m["rot"]["dims"], m["rot"]["base"], False)
+        kk = rotate(kk, pos, m["rot"]["dims"], m["rot"]["base"], False)
     rep = H // G
     kh = kk.repeat_interleave(rep, dim=1)
     vh = v.repeat_interleave(rep, dim=1)
     scores = torch.einsum("ihd,jhd->hij", q, kh) * m["scale"]
-    p = window_softmax(scores, m["mask"]["size"], w["sink"])
+    p = window_softmax(scores, window_of(m), w["sink"])
     o = torch.einsum("hij,jhd->ihd", p, vh).reshape(T, H * d)
     return o @ w["o"].T
 
@@ -92,12 +99,14 @@ def latent_attention(h: torch.Tensor, w: dict, m: dict, eps: float) -> torch.Ten
     c = rms(dkv[:, :rank], eps) * w["dkv.norm"]
     k_rot = dkv[:, rank:].view(T, 1, r)
     pos = torch.arange(T)
-    q_rot = rotate(q_rot, pos, r, m["rot"]["base"], True)
-    k_rot = rotate(k_rot, pos, r, m["rot"]["base"], True)[:, 0]
+    if r:
+        q_rot = rotate(q_rot, pos, r, m["rot"]["base"], True)
+        k_rot = rotate(k_rot, pos, r, m["rot"]["base"], True)
+    k_rot = k_rot[:, 0]
     k_plain = (c @ w["uk"].T).view(T, H, d)
     v = (c @ w["uv"].T).view(T, H, dv)
     scores = (torch.einsum("ihd,jhd->hij", q_plain, k_plain) + torch.einsum("ihd,jd->hij", q_rot, k_rot)) * m["scale"]
-    p = window_softmax(scores, m["mask"]["size"], None)
+    p = window_softmax(scores, window_of(m), None)
     o = torch.einsum("hij,jhd->ihd", p, v)
     gate = torch.sigmoid(h @ w["g"].T)
     return (o * gate[:, :, None]).reshape(T, H * dv) @ w["o"].T
@@ -165,3 +174,27 @@ def forward(config: dict, weights: dict, tokens: list[int], streams: list | None
     if cap:
         logits = cap * torch.tanh(logits / cap)
     return logits
+
+
+def load_model_folder(folder):
+    """``(config mapping, name -> float64 tensor)`` of a folder with config.json and safetensors files."""
+    import json
+    from pathlib import Path
+
+    from safetensors.torch import load_file
+
+    folder = Path(folder)
+    config = json.loads((folder / "config.json").read_text())
+    weights = {}
+    for file in sorted(folder.glob("*.safetensors")):
+        weights.update({k: v.to(F) for k, v in load_file(str(file)).items()})
+    return config, weights
+
+
+def windowed_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, window: int | None,
+                       sink: torch.Tensor | None) -> torch.Tensor:
+    """``q [T, H, d]``, ``k [T, G, d]``, ``v [T, G, dv]`` at positions 0..T-1 -> ``[T, H, dv]``."""
+    rep = q.shape[1] // k.shape[1]
+    kh, vh = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+    p = window_softmax(torch.einsum("ihd,jhd->hij", q, kh) * scale, window, sink)
+    return torch.einsum("hij,jhd->ihd", p, vh)
