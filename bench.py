@@ -20,7 +20,8 @@ Other workloads print a line of their own: ``--only-prefill``, ``--mixed`` (64 r
 with prompts of 16 to 2,048 tokens in portions of 512), ``--long-prompt N`` (time to the
 first token of one N-token prompt in portions of 2,048), ``--sweep`` (decode at further
 batch sizes and context lengths, a line each with its share of the memory bandwidth);
-``--model 1b|70b`` and ``--batch`` change the shape.  ``--vovalix s|m`` times the Vovalix
+``--model 1b|70b`` and ``--batch`` change the shape.  ``--tazunex s|m`` times the Tazunex
+decoder beside the Vovalix and the Llama of equal width and depth.  ``--vovalix s|m`` times the Vovalix
 decoder beside the Dirulorn of equal size.  ``--dirulorn s|m`` times the Dirulorn
 decoder (state-space layers beside attention-with-recurrence layers) at layer sizes of a real
 model, prefill and decode, next to a Llama of the same width, depth, feed-forward and head
@@ -116,6 +117,43 @@ VOVALIX_SHAPES = {
     "m": {"architecture": "Vovalix", "vocab": 32000, "width": 2048, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
           "layers": _vovalix_layers(16, 2048, 32, 8, 32, 4, 2048, 8, 4, 1024)},
 }
+
+
+def _tazunex_layers(n, width, heads, kv, ff, window):
+    dense = {"kind": "dense", "ff": ff}
+    rot = {"dims": 64, "base": 500000.0}
+    attention = {"type": "attention", "mlp": dense,
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 64, "scale": 0.125,
+                           "mask": {"size": window}, "rot": rot}}
+    latent = {"type": "latent_attention", "mlp": dense,
+              "mixer": {"heads": 16, "dim": width // 16, "rot_dim": 32, "vdim": width // 16, "kv_rank": 96,
+                        "q_rank": width // 2, "scale": 0.1, "mask": {"size": window},
+                        "rot": {"dims": 32, "base": 500000.0}}}
+    memory = {"type": "mlstm", "mlp": dense,
+              "mixer": {"heads": heads // 2, "dim": 64, "vdim": 128, "gate_cap": 15.0}}
+    return [(attention, memory, latent, memory)[i % 4] for i in range(n)]
+
+
+# Tazunex at the layer sizes of a real model: of every four layers one windowed attention with
+# sinks (keys of 64 that are the values too, windows of 1,024 positions), one latent attention
+# (sixteen heads on cached rows of 96 + 32 values, the same window) and two matrix memories (keys
+# of 64, values of 128), each before the dense gated feed-forward of the Llama of the same width
+TAZUNEX_SHAPES = {
+    "s": {"architecture": "Tazunex", "vocab": 32000, "width": 1024, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+          "layers": _tazunex_layers(8, 1024, 16, 4, 4096, 1024)},
+    "m": {"architecture": "Tazunex", "vocab": 32000, "width": 2048, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+          "layers": _tazunex_layers(16, 2048, 32, 8, 8192, 1024)},
+}
+
+
+def bench_tazunex(args) -> int:
+    """The workloads of ``bench_dirulorn`` for a Tazunex shape beside the Vovalix of the same width
+    and depth (the closest model the engine has: matrix-state recurrences beside attention that sees
+    a stretch of the sequence) and the Llama (the same dense feed-forward)."""
+    shapes = (TAZUNEX_SHAPES[args.tazunex], VOVALIX_SHAPES[args.tazunex], DIRULORN_SHAPES[args.tazunex][1])
+    names = (f"tazunex-{args.tazunex}", f"vovalix-of-tazunex-{args.tazunex}", f"llama-of-tazunex-{args.tazunex}")
+    which = {"all": (0, 1, 2), "tazunex": (0,), "vovalix": (1,), "llama": (2,)}[args.tazunex_only]
+    return _bench_design(args, shapes, names, which, args.tazunex_workload)
 
 
 def bench_vovalix(args) -> int:
@@ -251,6 +289,14 @@ def parse_args():
                    help="with --dirulorn: run one of the two models only (for profiling)")
     p.add_argument("--dirulorn-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
                    help="with --dirulorn: run one of the workloads only (for profiling)")
+    p.add_argument("--tazunex", default=None, choices=sorted(TAZUNEX_SHAPES),
+                   help="time the Tazunex decoder of this size (s: 8 layers of 1,024; m: 16 of 2,048) beside "
+                        "the Vovalix and the Llama of equal width and depth: prefill of 2,048 tokens, decode "
+                        "with 8 and 64 requests")
+    p.add_argument("--tazunex-only", default="all", choices=["all", "tazunex", "vovalix", "llama"],
+                   help="with --tazunex: run one of the models only (for profiling)")
+    p.add_argument("--tazunex-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
+                   help="with --tazunex: run one of the workloads only (for profiling)")
     p.add_argument("--vovalix", default=None, choices=sorted(VOVALIX_SHAPES),
                    help="instead of the headline line: prefill and decode of a Vovalix shape beside the "
                         "Dirulorn of the same width and depth; a line per model and workload")
@@ -408,6 +454,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.tazunex:
+        return bench_tazunex(args)
     if args.dirulorn:
         return bench_dirulorn(args)
     if args.vovalix:
