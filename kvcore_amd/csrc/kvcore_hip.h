@@ -219,13 +219,15 @@ int kvc_gated_group_rmsnorm(void* out, int out_dtype, const float* y, const void
 //   delta_rule 1:  S = decay[t, h] S;  u = beta[t, h] (v - S^T k);  S = S + k u^T
 //   delta_rule 2:  S = decay[t, h] S + beta[t, h] k v^T          (scalar gates per head)
 // and out[t, h] = S^T (q_scale q) after the token's write; out is [T, nh * dv] float32.  q, k, v, decay and
-// beta are float32 rows with strides.  d at most 256.
+// beta are float32 rows with strides.  d at most 256.  With ones_column the rows of v hold dv - 1
+// values a head and column dv - 1 of every head takes a one for each token: a normaliser that is
+// gated and read like the matrix, out[t, h, dv - 1] being its product with the query.
 int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const float* k,
                           int64_t k_stride, const float* v, int64_t v_stride, const float* decay,
                           int64_t decay_stride, const float* beta, int64_t beta_stride, float* state,
                           const int32_t* positions, const int32_t* token_req, const int32_t* q_start,
                           const int32_t* slots, int R, int nh, int nqk, int d, int dv, int delta_rule,
-                          float q_scale, kvc_stream stream);
+                          float q_scale, int ones_column, kvc_stream stream);
 // The gates of a matrix memory with log gates and a running maximum m (mLSTM), per request in
 // token order: i = cap tanh((i_raw + i_bias) / cap), f = logsigmoid(cap tanh((f_raw + f_bias) / cap)),
 // m_t = max(f + m_(t-1), i), keep[t, h] = exp(f + m_(t-1) - m_t), take[t, h] = exp(i - m_t),
@@ -234,15 +236,13 @@ int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const fl
 int kvc_max_gates(float* keep, float* take, float* m_out, const float* i_raw, int64_t i_stride,
                   const float* f_raw, int64_t f_stride, const float* i_bias, const float* f_bias,
                   float cap, float* m_state, const int32_t* positions, const int32_t* token_req,
-                  const int32_t* q_start, const int32_t* slots, int R, int nh, kvc_stream stream);
+                  const int32_t* q_start, const int32_t* slots, int T, int R, int nh,
+                  kvc_stream stream);
 // out[t, h, c] = y / sqrt(mean_c y^2 + eps) * gain[h * dv + c] * sigmoid(gate[t, h, c]) with
 // y = o[t, h, c] / (max(|o[t, h, dv]|, exp(-m[t, h])) + den_eps); o is [T, heads, dv + 1] float32.
 int kvc_max_gated_finish(void* out, int out_dtype, const float* o, const float* m, const void* gate,
                          int64_t gate_stride, int gate_dtype, const float* gain, float eps,
                          float den_eps, int T, int heads, int dv, kvc_stream stream);
-// out[t, h, :dv] = v[t, h, :], out[t, h, dv] = 1; out is [T, heads, dv + 1] float32.
-int kvc_append_ones(float* out, const float* v, int64_t v_stride, int T, int heads, int dv,
-                    kvc_stream stream);
 // a[t, i] = sigmoid(z[t, i] + bias[i]) ^ inv_tau, computed as exp(inv_tau * log sigmoid); bias may be null.
 int kvc_sigmoid_power(float* a, const float* z, int64_t z_stride, const float* bias, float inv_tau,
                       int T, int W, kvc_stream stream);

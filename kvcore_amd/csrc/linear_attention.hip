@@ -62,8 +62,11 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
     int64_t decay_stride, const float* __restrict__ beta, int64_t beta_stride, float* __restrict__ state,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots, int nh, int nqk, int d,
-    int dv, float q_scale, int scalar_gates) {
+    int dv, float q_scale, int scalar_gates, int ones_column) {
   constexpr int VT = 256 / NSL;  // value channels a block
+  // with ones_column the rows of v hold dv - 1 values a head and the last column of the state's dv
+  // takes a one for every token (a normaliser kept beside the matrix)
+  const int dvin = dv - ones_column;
   // FULL: d == NPT * NSL, so no row needs a bound, and a thread's rows of q, k and the factors lie
   // side by side in LDS (row n of a token at (n % NSL) * NPT + n / NSL), read 16 bytes at a time
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -217,7 +220,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       for (int j = 0; j < VN; ++j) {
         const int idx = tid + 256 * j, tt = idx / VT, cc = c0 + idx - tt * VT;
         const int64_t t = t0 + (tt < nt ? tt : 0);
-        vn[j] = cc < dv ? v[t * v_stride + h * dv + cc] : 0.f;
+        vn[j] = cc < dvin ? v[t * v_stride + h * dvin + cc] : (cc < dv ? 1.f : 0.f);
       }
     };
     auto stash = [&](float* base) {
@@ -278,7 +281,7 @@ __global__ __launch_bounds__(256) void linear_state_scan_kernel(
       }
       for (int idx = tid; idx < nt * VT; idx += nthreads) {
         const int tt = idx / VT, cc = c0 + idx - tt * VT;
-        v_s[idx] = cc < dv ? v[static_cast<int64_t>(t0 + tt) * v_stride + h * dv + cc] : 0.f;
+        v_s[idx] = cc < dvin ? v[static_cast<int64_t>(t0 + tt) * v_stride + h * dvin + cc] : (cc < dv ? 1.f : 0.f);
       }
       __syncthreads();
       work_stage(q_s, k_s, a_s, v_s, t0, nt);
@@ -357,59 +360,94 @@ __global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(
 // The log gates of a matrix memory with a running maximum (mLSTM), for every request's tokens in
 // order: i = cap tanh((i_raw + bi) / cap), f = logsigmoid(cap tanh((f_raw + bf) / cap)),
 // m_t = max(f_t + m_(t-1), i_t), keep_t = exp(f_t + m_(t-1) - m_t), take_t = exp(i_t - m_t).
-// A block a request: the gates of all its tokens side by side, then a thread a head walks the
-// maxima in order (an addition and a maximum a token), then the exponentials side by side.
-// m starts at 0 at position 0 and otherwise comes from the slot's state, where it goes back.
+// A wave a (request, head).  The step m -> max(m + f, i) composes: a run of tokens acts as
+// m -> max(m + A, B) with A the sum of its f and B the maximum it reaches from minus infinity.  So
+// each lane takes a run of consecutive tokens, finds its (A, B), the runs are joined lane by lane
+// from the request's m, and each lane walks its run again from where it starts: a chain of two
+// runs and 64 joins instead of one of all tokens.  m starts at 0 at position 0 and otherwise comes
+// from the slot's state, where the last one goes back.
+template <int GATES_MADE>
 __global__ __launch_bounds__(256) void max_gates_kernel(
     float* __restrict__ keep, float* __restrict__ take, float* __restrict__ m_out, const float* __restrict__ i_raw,
     int64_t i_stride, const float* __restrict__ f_raw, int64_t f_stride, const float* __restrict__ i_bias,
     const float* __restrict__ f_bias, float cap, float* __restrict__ m_state, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ token_req, const int32_t* __restrict__ q_start, const int32_t* __restrict__ slots,
     int nh) {
-  const int r = blockIdx.x, tid = threadIdx.x;
+  const int r = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int h_raw = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int h = h_raw < nh ? h_raw : nh - 1;  // a wave beyond the heads only keeps the barrier's count
   const int b = q_start[r], e = q_start[r + 1];
   if (e <= b) return;
-  const int n = (e - b) * nh;
+  const int n = e - b;
+  const int run = (n + kWave - 1) / kWave;
+  const int lo = b + (lane * run < n ? lane * run : n);
+  const int hi = b + ((lane + 1) * run < n ? (lane + 1) * run : n);
   if (token_req[b] < 0) {  // padding rows
-    for (int idx = tid; idx < n; idx += blockDim.x) {
-      keep[static_cast<int64_t>(b) * nh + idx] = 0.f;
-      take[static_cast<int64_t>(b) * nh + idx] = 0.f;
-      m_out[static_cast<int64_t>(b) * nh + idx] = 0.f;
+    for (int64_t t = lo; t < hi && h_raw < nh; ++t) {
+      keep[t * nh + h] = 0.f;
+      take[t * nh + h] = 0.f;
+      m_out[t * nh + h] = 0.f;
     }
     return;
   }
-  const float inv_cap = 1.f / cap;
-  for (int idx = tid; idx < n; idx += blockDim.x) {
-    const int tt = idx / nh, h = idx - tt * nh;
-    const int64_t t = b + tt;
-    const float gi = cap * tanhf((i_raw[t * i_stride + h] + i_bias[h]) * inv_cap);
-    const float gf = log_sigmoid_f(cap * tanhf((f_raw[t * f_stride + h] + f_bias[h]) * inv_cap));
-    take[t * nh + h] = gi;  // the log gates, until the maxima are known
-    keep[t * nh + h] = gf;
+  if (h_raw >= nh) {  // the whole wave
+    __syncthreads();
+    return;
   }
-  __syncthreads();
-  float* ms = m_state + static_cast<int64_t>(slots[r]) * nh;
-  const bool fresh = positions[b] == 0;
-  for (int h = tid; h < nh; h += blockDim.x) {
-    float m = fresh ? 0.f : ms[h];
-    for (int64_t t = b; t < e; ++t) {
-      // the maximum before this token goes where the token's own will stand: m_out[t] holds
-      // m_(t-1) until the pass below has read it
-      const float gf = keep[t * nh + h], gi = take[t * nh + h];
-      m_out[t * nh + h] = m;
-      m = fmaxf(gf + m, gi);
+  const float inv_cap = 1.f / cap, bi = i_bias[h], bf = f_bias[h];
+  // the log gates of all tokens first, dealt to the lanes one by one (nothing passes from token
+  // to token here, so the loads of several are in flight together); they stay in keep and take
+  // until the maxima are known
+  if (!GATES_MADE) {
+#pragma unroll 4
+    for (int64_t t = b + lane; t < e; t += kWave) {
+      take[t * nh + h] = cap * tanhf((i_raw[t * i_stride + h] + bi) * inv_cap);
+      keep[t * nh + h] = log_sigmoid_f(cap * tanhf((f_raw[t * f_stride + h] + bf) * inv_cap));
     }
-    ms[h] = m;
   }
-  __syncthreads();
-  for (int idx = tid; idx < n; idx += blockDim.x) {
-    const int64_t at = static_cast<int64_t>(b) * nh + idx;
-    const float gf = keep[at], gi = take[at], before = m_out[at];
-    const float m = fmaxf(gf + before, gi);  // the same operations as the walk's, so the same bits
-    keep[at] = expf(gf + before - m);
-    take[at] = expf(gi - m);
-    m_out[at] = m;
+  __syncthreads();  // the block's waves have one request: all of them arrive
+  float A = 0.f, B = -INFINITY;  // an empty run leaves m as it is
+#pragma unroll 4
+  for (int64_t t = lo; t < hi; ++t) {
+    const float gf = keep[t * nh + h], gi = take[t * nh + h];
+    A += gf;
+    B = fmaxf(B + gf, gi);
   }
+  float* ms = m_state + static_cast<int64_t>(slots[r]) * nh + h;
+  float m = positions[b] == 0 ? 0.f : *ms;
+  float mine = m;
+  for (int l = 0; l < kWave; ++l) {
+    if (l == lane) mine = m;
+    m = fmaxf(m + __shfl(A, l, kWave), __shfl(B, l, kWave));
+  }
+  if (lane == 0) *ms = m;
+  for (int64_t t = lo; t < hi; ++t) {
+    const float gf = keep[t * nh + h], gi = take[t * nh + h];
+    const float next = fmaxf(gf + mine, gi);
+    keep[t * nh + h] = expf(gf + mine - next);
+    take[t * nh + h] = expf(gi - next);
+    m_out[t * nh + h] = next;
+    mine = next;
+  }
+}
+
+// The log gates alone, a thread a (token, head): what max_gates_kernel<1> starts from.  With many
+// tokens a request the tanh, logarithm and exponential of every gate are most of the work, and
+// a wave a (request, head) would leave the chip idle.
+__global__ __launch_bounds__(256) void log_gates_kernel(float* __restrict__ keep, float* __restrict__ take,
+                                                         const float* __restrict__ i_raw, int64_t i_stride,
+                                                         const float* __restrict__ f_raw, int64_t f_stride,
+                                                         const float* __restrict__ i_bias,
+                                                         const float* __restrict__ f_bias, float cap, int64_t total,
+                                                         int nh) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t t = idx / nh;
+  const int h = static_cast<int>(idx - t * nh);
+  const float inv_cap = 1.f / cap;
+  take[idx] = cap * tanhf((i_raw[t * i_stride + h] + i_bias[h]) * inv_cap);
+  keep[idx] = log_sigmoid_f(cap * tanhf((f_raw[t * f_stride + h] + f_bias[h]) * inv_cap));
 }
 
 // The end of the same mixer: o[t, h, :dv] and the normaliser's product with the query at column dv
@@ -440,29 +478,27 @@ __global__ __launch_bounds__(256) void max_gated_finish_kernel(
     op[i] = from_float<TO>(p[i] / den * inv * gn[i] * sigmoid_f(to_float(gp[i])));
 }
 
-// v_out[t, h, :dv] = v[t, h, :], v_out[t, h, dv] = 1: the values with a column of ones, whose
-// column of the state is the normaliser.
-__global__ __launch_bounds__(256) void append_ones_kernel(float* __restrict__ out, const float* __restrict__ v,
-                                                          int64_t v_stride, int T, int heads, int dv) {
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int w = dv + 1;
-  if (idx >= static_cast<int64_t>(T) * heads * w) return;
-  const int64_t th = idx / w;
-  const int c = static_cast<int>(idx - th * w);
-  const int64_t t = th / heads;
-  const int h = static_cast<int>(th - t * heads);
-  out[idx] = c < dv ? v[t * v_stride + static_cast<int64_t>(h) * dv + c] : 1.f;
-}
-
 }  // namespace
 
 extern "C" int kvc_max_gates(float* keep, float* take, float* m_out, const float* i_raw, int64_t i_stride,
                              const float* f_raw, int64_t f_stride, const float* i_bias, const float* f_bias,
                              float cap, float* m_state, const int32_t* positions, const int32_t* token_req,
-                             const int32_t* q_start, const int32_t* slots, int R, int nh, kvc_stream stream) {
-  if (R < 0 || nh <= 0 || i_stride < nh || f_stride < nh || !(cap > 0.f)) return kvc_fail("kvc_max_gates: bad sizes");
-  if (R == 0) return 0;
-  hipLaunchKernelGGL(max_gates_kernel, dim3(R), dim3(256), 0, S(stream), keep, take, m_out, i_raw, i_stride, f_raw,
+                             const int32_t* q_start, const int32_t* slots, int T, int R, int nh,
+                             kvc_stream stream) {
+  if (T < 0 || R < 0 || nh <= 0 || i_stride < nh || f_stride < nh || !(cap > 0.f))
+    return kvc_fail("kvc_max_gates: bad sizes");
+  if (R == 0 || T == 0) return 0;
+  if (T > 2 * R) {  // portions of prompts: the gates by all threads first, then the walk of the maxima
+    const int64_t total = static_cast<int64_t>(T) * nh;
+    hipLaunchKernelGGL(log_gates_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, S(stream),
+                       keep, take, i_raw, i_stride, f_raw, f_stride, i_bias, f_bias, cap, total, nh);
+    hipLaunchKernelGGL(max_gates_kernel<1>, dim3(R, (nh + 3) / 4), dim3(256), 0, S(stream), keep, take, m_out, i_raw,
+                       i_stride, f_raw, f_stride, i_bias, f_bias, cap, m_state, positions, token_req, q_start, slots,
+                       nh);
+    return kvc_check_launch("kvc_max_gates");
+  }
+  // four waves a block, a wave a (request, head)
+  hipLaunchKernelGGL(max_gates_kernel<0>, dim3(R, (nh + 3) / 4), dim3(256), 0, S(stream), keep, take, m_out, i_raw, i_stride, f_raw,
                      f_stride, i_bias, f_bias, cap, m_state, positions, token_req, q_start, slots, nh);
   return kvc_check_launch("kvc_max_gates");
 }
@@ -493,24 +529,15 @@ extern "C" int kvc_max_gated_finish(void* out, int out_dtype, const float* o, co
   return kvc_check_launch("kvc_max_gated_finish");
 }
 
-extern "C" int kvc_append_ones(float* out, const float* v, int64_t v_stride, int T, int heads, int dv,
-                               kvc_stream stream) {
-  if (T < 0 || heads <= 0 || dv <= 0 || v_stride < static_cast<int64_t>(heads) * dv)
-    return kvc_fail("kvc_append_ones: bad sizes");
-  if (T == 0) return 0;
-  const int64_t n = static_cast<int64_t>(T) * heads * (dv + 1);
-  hipLaunchKernelGGL(append_ones_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, S(stream), out, v,
-                     v_stride, T, heads, dv);
-  return kvc_check_launch("kvc_append_ones");
-}
-
 extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_stride, const float* k,
                                      int64_t k_stride, const float* v, int64_t v_stride,
                                      const float* decay, int64_t decay_stride, const float* beta,
                                      int64_t beta_stride, float* state, const int32_t* positions,
                                      const int32_t* token_req, const int32_t* q_start,
                                      const int32_t* slots, int R, int nh, int nqk, int d, int dv,
-                                     int rule, float q_scale, kvc_stream stream) {
+                                     int rule, float q_scale, int ones_column,
+                                     kvc_stream stream) {
+  ones_column = ones_column ? 1 : 0;
   if (rule < 0 || rule > 2) return kvc_fail("kvc_linear_state_scan: the rule is 0 (key decay), 1 (delta) or 2 (scalar gates)");
   const int delta_rule = rule != 0;  // a gate and a factor per head and token instead of a decay per key channel
   const int scalar_gates = rule == 2;
@@ -520,7 +547,7 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   if (delta_rule && beta == nullptr) return kvc_fail("kvc_linear_state_scan: this rule needs beta");
   if (delta_rule && beta_stride < nh) return kvc_fail("kvc_linear_state_scan: rows of beta too short for the heads");
   if (q_stride < static_cast<int64_t>(nqk) * d || k_stride < static_cast<int64_t>(nqk) * d ||
-      v_stride < static_cast<int64_t>(nh) * dv || decay_stride < (delta_rule ? nh : static_cast<int64_t>(nh) * d))
+      v_stride < static_cast<int64_t>(nh) * (dv - ones_column) || dv - ones_column <= 0 || decay_stride < (delta_rule ? nh : static_cast<int64_t>(nh) * d))
     return kvc_fail("kvc_linear_state_scan: rows too short for the heads");
   if (R == 0) return 0;
   // tiles of 64 value channels with 4 threads a column, or, where that leaves compute units
@@ -537,7 +564,7 @@ extern "C" int kvc_linear_state_scan(float* out, const float* q, int64_t q_strid
   hipLaunchKernelGGL((linear_state_scan_kernel<NPT, DELTA, NSL_, FULL_, PF_>), grid, dim3(256),               \
                      lds*(PF_ ? 2 : 1), S(stream), out, q, q_stride, k, k_stride, v, v_stride, decay,         \
                      decay_stride, beta, beta_stride, state, positions, token_req, q_start, slots, nh, nqk, d, \
-                     dv, q_scale, scalar_gates)
+                     dv, q_scale, scalar_gates, ones_column)
   // two sets of LDS buffers (the next stage fetched while one is worked on) where a stage's values
   // deal out evenly to the threads and both sets fit the 64 KB a block may take
 #define KVC_LSCAN(NPT, DELTA, NSL_)                                                  \

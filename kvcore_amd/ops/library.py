@@ -46,16 +46,15 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, P],
         "kvc_wide_qk_norm": [P, L, P, P, F, I, I, I, I, I, P],
         "kvc_head_gate": [P, P, L, P, L, I, I, I, I, I, I, P],
-        "kvc_max_gates": [P, P, P, P, L, P, L, P, P, F, P, P, P, P, P, I, I, P],
+        "kvc_max_gates": [P, P, P, P, L, P, L, P, P, F, P, P, P, P, P, I, I, I, P],
         "kvc_max_gated_finish": [P, I, P, P, P, L, I, P, F, F, I, I, I, P],
-        "kvc_append_ones": [P, P, L, I, I, I, P],
         "kvc_gather_rows": [P, P, P, I, I, I, I, P],
         "kvc_to_float": [P, P, L, I, P],
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
         "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, I, P],
-        "kvc_linear_state_scan": [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, P],
+        "kvc_linear_state_scan": [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "kvc_sigmoid_power": [P, P, L, P, F, I, I, P],
         "kvc_decay_and_write_gates": [P, P, P, L, P, L, P, P, I, I, P],
         "kvc_unit_heads": [P, L, I, I, I, F, F, I, F, P],
@@ -1289,11 +1288,13 @@ def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
                       positions: torch.Tensor, token_req: torch.Tensor, q_start: torch.Tensor,
                       slots: torch.Tensor, num_reqs: int, heads: int, qk_heads: int, dim: int,
                       vdim: int, delta_rule: bool = False, q_scale: float = 1.0,
-                      scalar_gates: bool = False) -> None:
+                      scalar_gates: bool = False, ones_column: bool = False) -> None:
     """The recurrence of a matrix state per head (see the C header): ``q, k [T, qk_heads * dim]``,
     ``v [T, heads * vdim]``, all float32 rows (column views are fine); ``decay [T, heads * dim]``
     (a factor per key channel) or, with ``delta_rule``, ``decay`` and ``beta [T, heads]``; with
     ``scalar_gates`` the rule is ``S <- decay S + beta k v^T`` with the same two ``[T, heads]``;
+    with ``ones_column`` ``v`` is ``[T, heads * (vdim - 1)]`` and the last of a head's ``vdim``
+    columns takes a one for every token (a normaliser beside the matrix);
     ``state [slots, heads, linear_state_rows(dim), vdim]`` float32, in an order of the kernel's own;
     ``out [T, heads * vdim]`` float32.  ``q_scale``
     multiplies every q on its way in."""
@@ -1308,7 +1309,7 @@ def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
         raise KernelError("linear_state_scan: rows or index arrays too short")
     qp, qs = _f32_rows(q, "q", qk_heads * dim)
     kp, ks = _f32_rows(k, "k", qk_heads * dim)
-    vp, vs = _f32_rows(v, "v", heads * vdim)
+    vp, vs = _f32_rows(v, "v", heads * (vdim - 1 if ones_column else vdim))
     if delta_rule and scalar_gates:
         raise KernelError("linear_state_scan: one rule at a time")
     per_head = delta_rule or scalar_gates
@@ -1322,7 +1323,8 @@ def linear_state_scan(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
         out.data_ptr(), qp, qs, kp, ks, vp, vs, dp, ds, bp or None, bs, _dev(state, "state"),
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, heads,
-        qk_heads, dim, vdim, 2 if scalar_gates else int(bool(delta_rule)), float(q_scale), _stream()),
+        qk_heads, dim, vdim, 2 if scalar_gates else int(bool(delta_rule)), float(q_scale), int(bool(ones_column)),
+        _stream()),
         "kvc_linear_state_scan")
 
 
@@ -1397,7 +1399,7 @@ def max_gates(keep: torch.Tensor, take: torch.Tensor, m_out: torch.Tensor, i_raw
         _dev(keep, "keep", f), _dev(take, "take", f), _dev(m_out, "m_out", f), ip, is_, fp, fs,
         _dev(i_bias, "i_bias", f), _dev(f_bias, "f_bias", f), float(cap), _dev(m_state, "m_state", f),
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
-        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), num_reqs, nh, _stream()),
+        _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs, nh, _stream()),
         "kvc_max_gates")
 
 
@@ -1416,16 +1418,6 @@ def max_gated_finish(out: torch.Tensor, o: torch.Tensor, m: torch.Tensor, gate: 
         _dev(out, "out"), _code(out, "out"), _dev(o, "o", torch.float32), _dev(m, "m", torch.float32), gp, gs, gc,
         _dev(gain, "gain", torch.float32), float(eps), float(den_eps), T, heads, vdim, _stream()),
         "kvc_max_gated_finish")
-
-
-def append_ones(out: torch.Tensor, v: torch.Tensor, heads: int, vdim: int) -> None:
-    """``out [T, heads * (vdim + 1)]`` float32: every head's ``vdim`` values of ``v`` (float32 rows, a
-    column view is fine) and a one behind them."""
-    T = out.shape[0]
-    if out.shape != (T, heads * (vdim + 1)) or not out.is_contiguous() or out.dtype != torch.float32 or v.shape[0] < T:
-        raise KernelError("append_ones: shapes do not match")
-    vp, vs = _f32_rows(v, "v", heads * vdim)
-    _check(load().kvc_append_ones(out.data_ptr(), vp, vs, T, heads, vdim, _stream()), "kvc_append_ones")
 
 
 def norm_add_norm(out: torch.Tensor | None, residual: torch.Tensor, delta: torch.Tensor,

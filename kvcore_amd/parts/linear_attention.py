@@ -254,11 +254,10 @@ class MaxGatedMatrixMemory(_MatrixStateMixer):
         ops.max_gates(keep, take, m, proj[:, at:at + nh], proj[:, at + nh:], p["i.bias"], p["f.bias"], self.cap,
                       maxima, **batch)
         wide = nh * (self.vdim + 1)
-        v1 = ctx.buf(f"mm_v:{wide}", wide, torch.float32)
-        ops.append_ones(v1, proj[:, 2 * qk:2 * qk + inner], nh, self.vdim)
         o = ctx.buf(f"mm_o:{wide}", wide, torch.float32)
-        ops.linear_state_scan(o, proj[:, :qk], proj[:, qk:2 * qk], v1, keep, take, state, heads=nh, qk_heads=nh,
-                              dim=self.dim, vdim=self.vdim + 1, scalar_gates=True, q_scale=self.q_scale, **batch)
+        ops.linear_state_scan(o, proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + inner], keep, take, state,
+                              heads=nh, qk_heads=nh, dim=self.dim, vdim=self.vdim + 1, scalar_gates=True,
+                              ones_column=True, q_scale=self.q_scale, **batch)
         normed = ctx.buf(f"ms_normed:{inner}", inner)
         ops.max_gated_finish(normed, o, m, proj[:, 2 * qk + inner:2 * qk + 2 * inner], p["norm"], self.eps,
                              self.den_eps, nh, self.vdim)

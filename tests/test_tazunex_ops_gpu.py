@@ -143,11 +143,10 @@ def run_memory(h, w, m, state, maxima, reqs, eps):
     at = 2 * qk + 2 * inner
     ops.max_gates(keep, take, mx, proj[:, at:at + H], proj[:, at + H:], gpu(w["i.b"]), gpu(w["f.b"]), m["gate_cap"],
                   maxima, **batch)
-    v1 = torch.full((T, H * (dv + 1)), float("nan"), device=DEV)
-    ops.append_ones(v1, proj[:, 2 * qk:2 * qk + inner], H, dv)
     o = torch.full((T, H * (dv + 1)), float("nan"), device=DEV)
-    ops.linear_state_scan(o, proj[:, :qk], proj[:, qk:2 * qk], v1, keep, take, state, heads=H, qk_heads=H, dim=d,
-                          vdim=dv + 1, scalar_gates=True, q_scale=d ** -0.5, **batch)
+    ops.linear_state_scan(o, proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + inner], keep, take, state,
+                          heads=H, qk_heads=H, dim=d, vdim=dv + 1, scalar_gates=True, ones_column=True,
+                          q_scale=d ** -0.5, **batch)
     out = torch.full((T, inner), float("nan"), device=DEV)
     ops.max_gated_finish(out, o, mx, proj[:, 2 * qk + inner:at], gpu(w["norm"]), eps, 1e-6, H, dv)
     return out
