@@ -356,6 +356,12 @@ int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* del
 // are copied behind them first (values that are the keys as projected).
 int kvc_wide_qk_norm(void* qkv, int64_t stride, const float* q_gain, const float* k_gain, float eps,
                      int T, int nq, int nk, int copy_k, int dtype, kvc_stream stream);
+// Rows of down are [q_rank | rank | rot | ...]: cq[t] = q_gain * rms-normed first run; key[t] and
+// value[t] (rows kv_stride apart) both receive [the rot values as they are | kv_gain * rms-normed
+// second run]: what a latent attention caches a token, laid out with the rotated part first.
+int kvc_latent_rows(void* cq, int64_t cq_stride, void* key, void* value, int64_t kv_stride, const void* down,
+                    int64_t down_stride, const float* q_gain, const float* kv_gain, float eps, int T,
+                    int q_rank, int rank, int rot, int dtype, kvc_stream stream);
 // out[t, h * n + e] = x[t * x_stride + h * head_stride + skip + e] * sigmoid(gate[t * gate_stride + h]),
 // e < n: a gate per head, and a run of each head's columns kept.  gate has the dtype of x and out.
 int kvc_head_gate(void* out, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,

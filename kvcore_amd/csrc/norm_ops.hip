@@ -5,6 +5,7 @@
 // into the float32 stream and the norm of the new stream: one block a row does all three with
 // the row in registers (rows of a multiple of 8 values up to 16,384), or from memory otherwise.
 // kvc_wide_qk_norm: the query and key norms of an attention whose norm spans all heads at once.
+// kvc_latent_rows: the two latent norms of a latent attention and its one key/value row a token.
 // kvc_head_gate: a sigmoid gate per head on a run of each head's columns.
 // Sums of squares, scale factors and the stream are float32 whatever the storage type.
 
@@ -174,6 +175,48 @@ __global__ __launch_bounds__(256) void wide_qk_norm_kernel(T* __restrict__ qkv, 
     row[nq + i] = from_float<T>(k_gain[i] * (to_float(row[nq + i]) * inv_k));
 }
 
+// One block a token: what a latent attention makes of its down projection.  Rows of `down` hold
+// [query latent of q_rank | key/value latent of rank | rot rotated key elements | ...]: the query
+// latent, normed with q_gain, goes to cq; the row [rotated elements as they are | latent normed
+// with kv_gain] goes to `key` and, the same values, to `value` (the one row a token that the cache
+// keeps, in the place of a key and in the place of a value).
+template <typename T>
+__global__ __launch_bounds__(256) void latent_rows_kernel(T* __restrict__ cq, int64_t cq_stride, T* __restrict__ key,
+                                                          T* __restrict__ value, int64_t kv_stride,
+                                                          const T* __restrict__ down, int64_t down_stride,
+                                                          const float* __restrict__ q_gain,
+                                                          const float* __restrict__ kv_gain, float eps, int q_rank,
+                                                          int rank, int rot) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const T* row = down + t * down_stride;
+  float sq = 0.f, sc = 0.f;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
+    const float v = to_float(row[i]);
+    sq += v * v;
+  }
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const float v = to_float(row[q_rank + i]);
+    sc += v * v;
+  }
+  const float inv_q = rsqrtf(block_sum(sq, scratch) / static_cast<float>(q_rank) + eps);
+  const float inv_c = rsqrtf(block_sum(sc, scratch) / static_cast<float>(rank) + eps);
+  T* q_out = cq + t * cq_stride;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) q_out[i] = from_float<T>(q_gain[i] * (to_float(row[i]) * inv_q));
+  T* k_out = key + t * kv_stride;
+  T* v_out = value + t * kv_stride;
+  for (int i = threadIdx.x; i < rot; i += blockDim.x) {
+    const T raw = row[q_rank + rank + i];
+    k_out[i] = raw;
+    v_out[i] = raw;
+  }
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const T c = from_float<T>(kv_gain[i] * (to_float(row[q_rank + i]) * inv_c));
+    k_out[rot + i] = c;
+    v_out[rot + i] = c;
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t x_stride,
                                                         const T* __restrict__ gate, int64_t gate_stride,
@@ -226,6 +269,23 @@ extern "C" int kvc_wide_qk_norm(void* qkv, int64_t stride, const float* q_gain, 
                      hipLaunchKernelGGL(wide_qk_norm_kernel<Tp>, dim3(T), dim3(256), 0, S(stream),
                                         static_cast<Tp*>(qkv), stride, q_gain, k_gain, eps, nq, nk, copy_k));
   return kvc_check_launch("kvc_wide_qk_norm");
+}
+
+extern "C" int kvc_latent_rows(void* cq, int64_t cq_stride, void* key, void* value, int64_t kv_stride,
+                               const void* down, int64_t down_stride, const float* q_gain, const float* kv_gain,
+                               float eps, int T, int q_rank, int rank, int rot, int dtype, kvc_stream stream) {
+  if (T < 0 || q_rank <= 0 || rank <= 0 || rot < 0 || cq_stride < q_rank || kv_stride < rank + rot ||
+      down_stride < static_cast<int64_t>(q_rank) + rank + rot)
+    return kvc_fail("kvc_latent_rows: rows too short for the sections");
+  if (cq == nullptr || key == nullptr || value == nullptr || down == nullptr || q_gain == nullptr || kv_gain == nullptr)
+    return kvc_fail("kvc_latent_rows: null operand");
+  if (T == 0) return 0;
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(latent_rows_kernel<Tp>, dim3(T), dim3(256), 0, S(stream), static_cast<Tp*>(cq),
+                                        cq_stride, static_cast<Tp*>(key), static_cast<Tp*>(value), kv_stride,
+                                        static_cast<const Tp*>(down), down_stride, q_gain, kv_gain, eps, q_rank, rank,
+                                        rot));
+  return kvc_check_launch("kvc_latent_rows");
 }
 
 extern "C" int kvc_head_gate(void* out, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,

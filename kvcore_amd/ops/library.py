@@ -46,6 +46,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, P],
         "kvc_wide_qk_norm": [P, L, P, P, F, I, I, I, I, I, P],
         "kvc_head_gate": [P, P, L, P, L, I, I, I, I, I, I, P],
+        "kvc_latent_rows": [P, L, P, P, L, P, L, P, P, F, I, I, I, I, I, P],
         "kvc_max_gates": [P, P, P, P, L, P, L, P, P, F, P, P, P, P, P, I, I, I, P],
         "kvc_max_gated_finish": [P, I, P, P, P, L, I, P, F, F, I, I, I, P],
         "kvc_gather_rows": [P, P, P, I, I, I, I, P],
@@ -1453,6 +1454,25 @@ def wide_qk_norm(qkv: torch.Tensor, q_gain: torch.Tensor, k_gain: torch.Tensor, 
     _check(load().kvc_wide_qk_norm(qkv.data_ptr(), qkv.stride(0), _dev(q_gain, "q_gain", torch.float32),
                                    _dev(k_gain, "k_gain", torch.float32), float(eps), qkv.shape[0], nq, nk,
                                    int(bool(copy_k)), _code(qkv, "qkv"), _stream()), "kvc_wide_qk_norm")
+
+
+def latent_rows(cq: torch.Tensor, key: torch.Tensor, value: torch.Tensor, down: torch.Tensor, q_gain: torch.Tensor,
+                kv_gain: torch.Tensor, eps: float, rot: int) -> None:
+    """From rows ``down = [query latent | key/value latent | rot rotated key elements | ...]``: the
+    query latent normed with ``q_gain`` into ``cq``; ``[rotated elements as they are | key/value
+    latent normed with kv_gain]`` into ``key`` and into ``value`` (column views of one buffer with
+    equal row strides are fine).  All of one dtype; the norms are float32."""
+    T = down.shape[0]
+    q_rank, rank = q_gain.numel(), kv_gain.numel()
+    for t, cols in ((cq, q_rank), (key, rank + rot), (value, rank + rot)):
+        if t.dim() != 2 or t.shape != (T, cols) or t.stride(1) != 1 or t.dtype != down.dtype:
+            raise KernelError("latent_rows: results do not fit")
+    if down.stride(1) != 1 or down.shape[1] < q_rank + rank + rot or key.stride(0) != value.stride(0):
+        raise KernelError("latent_rows: rows too short, or keys and values with different strides")
+    _check(load().kvc_latent_rows(cq.data_ptr(), cq.stride(0), key.data_ptr(), value.data_ptr(), key.stride(0),
+                                  down.data_ptr(), down.stride(0), _dev(q_gain, "q_gain", torch.float32),
+                                  _dev(kv_gain, "kv_gain", torch.float32), float(eps), T, q_rank, rank, int(rot),
+                                  _code(down, "down"), _stream()), "kvc_latent_rows")
 
 
 def head_gate(out: torch.Tensor, x: torch.Tensor, gate: torch.Tensor, *, heads: int, head_stride: int,

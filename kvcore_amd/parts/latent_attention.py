@@ -107,16 +107,12 @@ class LatentAttention(PagedAttention):
         down = ctx.buf(f"latent_down:{self.down_width}", self.down_width)
         ops.linear(down, x, p["down.weight"])
         cq = ctx.buf(f"latent_cq:{self.q_rank}", self.q_rank)
-        ops.rmsnorm(cq, down[:, : self.q_rank], p["dq_norm"], self.eps)
         qkv = ctx.buf(f"latent_qkv:{(nh + 2) * row}", (nh + 2) * row)
+        # both latents' norms and the one key/value row a token (the rotated part as projected,
+        # then the normed latent; the same values in the key's place and in the value's)
+        ops.latent_rows(cq, qkv[:, nh * row: (nh + 1) * row], qkv[:, (nh + 1) * row:], down, p["dq_norm"],
+                        p["dkv_norm"], self.eps, rot)
         ops.linear(qkv[:, : nh * row], cq, p["q_latent.weight"])
-        # the one key/value row a token: the rotated part as projected, then the normed latent
-        key = qkv[:, nh * row: (nh + 1) * row]
-        at = self.q_rank
-        if rot:
-            key[:, :rot].copy_(down[:, at + rank: at + rank + rot])
-        ops.rmsnorm(key[:, rot:], down[:, at: at + rank], p["dkv_norm"], self.eps)
-        qkv[:, (nh + 1) * row:].copy_(key)
         ctx.scratch[("latent_down", id(self))] = down
         return qkv
 

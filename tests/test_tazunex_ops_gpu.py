@@ -86,6 +86,31 @@ def test_gate_per_head_on_a_run_of_columns(dtype):
     assert rel(out, want.reshape(T, -1)) < (1e-6 if dtype == torch.float32 else 4e-3)
 
 
+@pytest.mark.parametrize("q_rank,rank,rot,extra", [(40, 24, 8, 3), (1, 6, 2, 1), (7, 5, 0, 2), (1024, 96, 32, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_latent_norms_and_the_cached_row(q_rank, rank, rot, extra, dtype):
+    """The query latent and the key/value latent each over its own root mean square; the cached
+    row is the rotated part as projected (not normed), then the normed latent, twice."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(q_rank + rank)
+    T, eps, heads = 13, 1e-5, 3
+    down = (torch.randn(T, q_rank + rank + rot + extra, generator=gen, dtype=F64) * 2).to(dtype).double()
+    down[:, q_rank:q_rank + rank] *= 4  # the two latents differ in size, so one norm over both would show
+    gq, gc = 1 + 0.3 * torch.randn(q_rank, generator=gen, dtype=F64), 1 + 0.3 * torch.randn(rank, generator=gen, dtype=F64)
+    row = rot + rank
+    cq = torch.full((T, q_rank), float("nan"), dtype=dtype, device=DEV)
+    qkv = torch.full((T, (heads + 2) * row), float("nan"), dtype=dtype, device=DEV)
+    ops.latent_rows(cq, qkv[:, heads * row:(heads + 1) * row], qkv[:, (heads + 1) * row:], gpu(down, dtype), gpu(gq),
+                    gpu(gc), eps, rot)
+    tol = 1e-6 if dtype == torch.float32 else 4e-3
+    assert rel(cq, plain.rms(down[:, :q_rank], eps) * gq) < tol
+    want = torch.cat([down[:, q_rank + rank:q_rank + rank + rot], plain.rms(down[:, q_rank:q_rank + rank], eps) * gc], dim=1)
+    assert rel(qkv[:, heads * row:(heads + 1) * row], want) < tol
+    assert torch.equal(qkv[:, heads * row:(heads + 1) * row], qkv[:, (heads + 1) * row:])
+    assert torch.isnan(qkv[:, :heads * row]).all()  # the queries' place is left alone
+
+
 # ------------------------------------------------------------------ the gated feed-forward
 @pytest.mark.parametrize("dtype,M,H,I", [(torch.float32, 9, 40, 24), (torch.bfloat16, 1, 64, 48), (torch.bfloat16, 16, 128, 136),
                                          (torch.bfloat16, 40, 512, 256), (torch.bfloat16, 150, 1024, 128),
