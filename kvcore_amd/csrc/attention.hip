@@ -1,7 +1,7 @@
 // Paged attention, general kernel: one 64-lane wave per (token, query head).
 //
 // Serves every batch shape (portions of prompts beside single decoded tokens), both
-// storage types and every head size that is a multiple of 16 up to 256.  A token at
+// storage types and every head size up to 512 (heads above 256 in instances of their own).  A token at
 // position p reads keys first..p of its request through the block table, 64 keys a
 // tile: each lane scores one key (a float32 dot product over the head in index
 // order), the tile is folded into a running softmax (float32 max, sum and output
@@ -23,7 +23,8 @@ using namespace kvc;
 namespace {
 
 constexpr int kWavesPerBlock = 4;
-constexpr int kMaxHeadDim = 256;
+constexpr int kMaxHeadDim = 512;    // the widest head served
+constexpr int kUsualHeadDim = 256;  // heads up to this size take the instances with half the registers
 
 template <typename T>
 struct Vec16;  // 16 bytes of T
@@ -43,14 +44,14 @@ struct Vec16<bf16_t> {
   }
 };
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_kernel(
     T* __restrict__ out, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int32_t* __restrict__ table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ slots, int nh, int nkv, int d, int dv, int page_size, int num_pages,
     float scale, int window, const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks) {
-  __shared__ float q_s[kWavesPerBlock][kMaxHeadDim];
+  __shared__ float q_s[kWavesPerBlock][MAXD];
   __shared__ float p_s[kWavesPerBlock][kWave];
   __shared__ int64_t off_s[kWavesPerBlock][kWave];   // K row of each key of the tile
   __shared__ int64_t voff_s[kWavesPerBlock][kWave];  // V column of each key of the tile
@@ -88,9 +89,9 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     m = sinks[h];
     l = 1.f;
   }
-  float acc[kMaxHeadDim / kWave];
+  float acc[MAXD / kWave];
 #pragma unroll
-  for (int i = 0; i < kMaxHeadDim / kWave; ++i) acc[i] = 0.f;
+  for (int i = 0; i < MAXD / kWave; ++i) acc[i] = 0.f;
 
   constexpr int VN = Vec16<T>::N;
   const int64_t head_off = static_cast<int64_t>(hk) * page_size * d;
@@ -138,14 +139,14 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     __syncthreads();
     const int n_keys = (pos - tile + 1 < kWave) ? pos - tile + 1 : kWave;
 #pragma unroll
-    for (int i = 0; i < kMaxHeadDim / kWave; ++i) acc[i] *= alpha;
+    for (int i = 0; i < MAXD / kWave; ++i) acc[i] *= alpha;
     for (int j = 0; j < n_keys; ++j) {
       const int64_t vo = voff_s[wave][j];
       if (vo < 0) continue;
       const float pj = p_s[wave][j];
       const T* vr = v_cache + vo;  // element e of this key is at vr[e * page_size]
 #pragma unroll
-      for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+      for (int i = 0; i < MAXD / kWave; ++i) {
         const int e = lane + i * kWave;
         if (e < dv) acc[i] = fmaf(pj, to_float(vr[static_cast<int64_t>(e) * page_size]), acc[i]);
       }
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
   if (!head_live) return;
   const float inv = (l > 0.f) ? 1.f / l : 0.f;
 #pragma unroll
-  for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+  for (int i = 0; i < MAXD / kWave; ++i) {
     const int e = lane + i * kWave;
     if (e < dv) o[e] = from_float<T>(acc[i] * inv);
   }
@@ -173,16 +174,27 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
     return kvc_fail("kvc_paged_attention: bad sizes");
   if (nh % nkv) return kvc_fail("kvc_paged_attention: heads must be a multiple of kv heads");
   if (d <= 0 || d > kMaxHeadDim)
-    return kvc_fail("kvc_paged_attention: head size must be positive, at most 256");
+    return kvc_fail("kvc_paged_attention: head size must be positive, at most 512");
   if (dv <= 0 || dv > kMaxHeadDim)
-    return kvc_fail("kvc_paged_attention: value size must be positive, at most 256");
+    return kvc_fail("kvc_paged_attention: value size must be positive, at most 512");
   if (q_stride < static_cast<int64_t>(nh) * d)
     return kvc_fail("kvc_paged_attention: q stride too small");
   if (T == 0) return 0;
   const dim3 grid(T, (nh + kWavesPerBlock - 1) / kWavesPerBlock);
+  if (d > kUsualHeadDim || dv > kUsualHeadDim) {
+    KVC_DISPATCH_DTYPE(
+        dtype, Tp,
+        hipLaunchKernelGGL((paged_attention_wave_kernel<Tp, kMaxHeadDim>), grid, dim3(kWavesPerBlock * kWave), 0,
+                           reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(out),
+                           static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
+                           static_cast<const Tp*>(v_cache), table, table_stride, positions,
+                           token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window, slopes,
+                           chunk, sinks));
+    return kvc_check_launch("kvc_paged_attention");
+  }
   KVC_DISPATCH_DTYPE(
       dtype, Tp,
-      hipLaunchKernelGGL(paged_attention_wave_kernel<Tp>, grid, dim3(kWavesPerBlock * kWave), 0,
+      hipLaunchKernelGGL((paged_attention_wave_kernel<Tp, kUsualHeadDim>), grid, dim3(kWavesPerBlock * kWave), 0,
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(out),
                          static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
                          static_cast<const Tp*>(v_cache), table, table_stride, positions,
@@ -206,14 +218,14 @@ struct ValuePlanes {
   T* plane[kMaxValuePlanes];
 };
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     T* __restrict__ qkv, int64_t row_stride, T* __restrict__ k_cache, ValuePlanes<T> v_planes, int v_chunk,
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
     const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim,
     int interleaved, const int32_t* __restrict__ kv_slot, int nh, int nkv, int d, int dv,
     int page_size, int write_kv, int copy_values) {
-  __shared__ float head_s[4][kMaxHeadDim];
+  __shared__ float head_s[4][MAXD];
   const int t = blockIdx.x;
   const int slot = kv_slot[t];
   if (slot == -2) return;  // padding token
@@ -233,10 +245,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     const int head = live ? head_base + wave : 0;
     T* hp = row + static_cast<int64_t>(head) * d;
     const float* gain = head < nh ? q_gain : k_gain;
-    float x[kMaxHeadDim / kWave];
+    float x[MAXD / kWave];
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+    for (int i = 0; i < MAXD / kWave; ++i) {
       const int e = lane + i * kWave;
       x[i] = e < d ? to_float(hp[e]) : 0.f;
       ss = fmaf(x[i], x[i], ss);
@@ -245,13 +257,13 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
       ss = wave_sum(ss);
       const float inv = 1.f / sqrtf(ss / static_cast<float>(d) + eps);
 #pragma unroll
-      for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+      for (int i = 0; i < MAXD / kWave; ++i) {
         const int e = lane + i * kWave;
         if (e < d) x[i] = x[i] * inv * gain[e];
       }
     }
 #pragma unroll
-    for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+    for (int i = 0; i < MAXD / kWave; ++i) {
       const int e = lane + i * kWave;
       if (e < d) head_s[wave][e] = x[i];
     }
@@ -260,7 +272,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kv_write_kernel(
     if (live && head >= nh && store_kv)
       kc = k_cache + ((static_cast<int64_t>(page) * nkv + (head - nh)) * page_size + off) * d;
 #pragma unroll
-    for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
+    for (int i = 0; i < MAXD / kWave; ++i) {
       const int e = lane + i * kWave;
       if (e >= d || !live) continue;
       float y = x[i];
@@ -398,7 +410,7 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
                                          int dtype, kvc_stream stream) {
   if (T < 0 || nh <= 0 || nkv <= 0 || d <= 0 || dv <= 0 || page_size <= 0)
     return kvc_fail("kvc_qk_norm_rope_kv_write: bad sizes");
-  if (d > kMaxHeadDim) return kvc_fail("kvc_qk_norm_rope_kv_write: head size above 256");
+  if (d > kMaxHeadDim) return kvc_fail("kvc_qk_norm_rope_kv_write: head size above 512");
   if (rot_dim < 0 || rot_dim > d || (rot_dim & 1))
     return kvc_fail("kvc_qk_norm_rope_kv_write: rot_dim must be even and at most the head size");
   if (row_stride < static_cast<int64_t>(nh + nkv) * d + static_cast<int64_t>(nkv) * dv)
@@ -433,10 +445,25 @@ extern "C" int kvc_qk_norm_rope_kv_write(void* qkv, int64_t row_stride, void* k_
                            planes, v_chunk, kv_slot, T, (nh + nkv) * d, nkv, dv, page_size));
     return kvc_check_launch("kvc_qk_norm_rope_kv_write");
   }
+  if (d > kUsualHeadDim) {
+    KVC_DISPATCH_DTYPE(
+        dtype, Tp, ValuePlanes<Tp> planes{};
+        for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);
+        hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<Tp, kMaxHeadDim>), dim3(T, head_groups), dim3(256), 0,
+                           reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv), row_stride,
+                           static_cast<Tp*>(k_cache), planes, v_chunk, q_gain, k_gain, eps,
+                           cos_tab, sin_tab, rot_dim, interleaved, kv_slot, nh, nkv, d, dv, page_size,
+                           write_kv, tiled_values ? 0 : 1);
+        if (tiled_values) hipLaunchKernelGGL(
+            value_planes_write_tile_kernel<Tp>, dim3((T + 7) / 8), dim3(256), 0,
+            reinterpret_cast<hipStream_t>(stream), static_cast<const Tp*>(qkv), row_stride, planes,
+            v_chunk, kv_slot, T, (nh + nkv) * d, nkv, dv, page_size));
+    return kvc_check_launch("kvc_qk_norm_rope_kv_write");
+  }
   KVC_DISPATCH_DTYPE(
       dtype, Tp, ValuePlanes<Tp> planes{};
       for (int c = 0; c < num_v_planes; ++c) planes.plane[c] = static_cast<Tp*>(host_v_planes[c]);
-      hipLaunchKernelGGL(qk_norm_rope_kv_write_kernel<Tp>, dim3(T, head_groups), dim3(256), 0,
+      hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<Tp, kUsualHeadDim>), dim3(T, head_groups), dim3(256), 0,
                          reinterpret_cast<hipStream_t>(stream), static_cast<Tp*>(qkv), row_stride,
                          static_cast<Tp*>(k_cache), planes, v_chunk, q_gain, k_gain, eps,
                          cos_tab, sin_tab, rot_dim, interleaved, kv_slot, nh, nkv, d, dv, page_size,

@@ -146,8 +146,8 @@ class PagedAttention(Mixer):
             if qk_norm_eps is None and not values_are_keys and not self.any_head_size:
                 raise ValueError(f"head size {head_dim} is not supported (multiples of 16 up to 256)")
             plain = False  # the kernel that rotates and writes heads of any size, and the general attention
-        if not 0 < head_dim <= 256 or not 0 < v_head_dim <= 256:
-            raise ValueError(f"head sizes {head_dim} and {v_head_dim} are not supported (1 to 256)")
+        if not 0 < head_dim <= 512 or not 0 < v_head_dim <= 512:
+            raise ValueError(f"head sizes {head_dim} and {v_head_dim} are not supported (1 to 512)")
         self.hidden_size = hidden_size
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads

@@ -43,9 +43,9 @@ class LatentAttention(PagedAttention):
         if min(heads, dim, vdim, kv_rank, q_rank) <= 0 or rot_dim < 0 or rot_dim % 2:
             raise ValueError("latent attention needs positive sizes and an even rotated width")
         width = rot_dim + kv_rank
-        if width > 256:
+        if width > 512:
             raise ValueError(f"a latent of {kv_rank} with {rot_dim} rotated elements: the attention kernels "
-                             f"serve rows of up to 256 values")
+                             f"serve rows of up to 512 values")
         super().__init__(hidden_size=hidden_size, num_heads=heads, num_kv_heads=1, head_dim=width, scale=scale,
                          window=window, page_size=page_size, float32_result=float32_result, position=position)
         self.heads, self.dim, self.rot, self.vdim = heads, dim, rot_dim, vdim

@@ -88,13 +88,15 @@ CONFIG_C = {
 
 # wide states and many heads: 200 key channels a head (many rows a thread), 80 value channels
 # (with the normaliser's column more than one tile), twenty query heads on one latent row of 64
-# (more than the kernel for single tokens takes a kv head), heads of 48 rotated whole
+# (more than the kernel for single tokens takes a kv head), heads of 48 rotated whole, a latent of
+# 280 values (cached rows of 288: wider than the attention kernels' usual instances)
 CONFIG_D = {
     "architecture": "Tazunex", "vocab": 256, "width": 64, "norm": {"eps": 1e-6}, "logit_softcap": 10.0,
     "layers": [
         {"type": "mlstm", "mixer": _mem(2, 200, 80, 5.0), "mlp": _ff(32)},
         {"type": "latent_attention", "mixer": _latent(20, 16, 16, 8, 48, 24, 0.15, 70), "mlp": _ff(32)},
         {"type": "attention", "mixer": _attn(3, 1, 48, 0.15, 100, (48, 25000.0)), "mlp": None},
+        {"type": "latent_attention", "mixer": _latent(2, 24, 8, 16, 280, 32, 0.1, 40), "mlp": None},
     ],
 }
 
