@@ -274,7 +274,7 @@ def parse_args():
                         "(default: where the device has room, as the engine decides)")
     p.add_argument("--sampling", default=None, metavar="T[,K[,P]]",
                    help="sample with this temperature, top-k and top-p (seeded) instead of greedily; "
-                        "not the contract's line: say so with --no-points")
+                        "not the default greedy line: say so with --no-points")
     p.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     p.add_argument("--only-prefill", action="store_true",
                    help="run only the 2,048-token prefill (for profiling); prints its own line")
@@ -523,7 +523,7 @@ def main() -> int:
     sampling = {"temperature": 0.0}
     if args.sampling:
         if not args.no_points:
-            print("bench.py: --sampling is not the contract's greedy line; pass --no-points with it", file=sys.stderr)
+            print("bench.py: --sampling is not the default greedy line; pass --no-points with it", file=sys.stderr)
             return 2
         parts = [float(v) for v in args.sampling.split(",")]
         sampling = {"temperature": parts[0], "seed": 1}

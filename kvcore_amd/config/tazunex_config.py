@@ -157,27 +157,37 @@ class TazunexConfig:
         raw_layers = d.get("layers")
         if not isinstance(raw_layers, list) or not raw_layers:
             raise ConfigError("config.json: 'layers' must be a list of at least one layer")
-        layers: list[TazunexLayerConfig] = []
         for i, raw in enumerate(raw_layers):
-            where = f"layers[{i}]."
             if not isinstance(raw, Mapping):
                 raise ConfigError(f"config.json: layers[{i}] must be an object")
+        slots: list[TazunexLayerConfig | None] = [None] * len(raw_layers)
+        for i, raw in enumerate(raw_layers):  # the layers that own tensors
+            if raw.get("weights_of") is not None:
+                continue
+            where = f"layers[{i}]."
             kind = raw.get("type")
             if kind not in _MIXERS:
                 raise ConfigError(f"config.json: {where}type {kind!r} is not supported (supported: {sorted(_MIXERS)})")
-            source = raw.get("weights_of")
-            if source is None:
-                mixer = _MIXERS[kind].from_dict(_mapping(raw, "mixer", where), where + "mixer.")
-                mlp = None if raw.get("mlp") is None else DenseFeedForwardConfig.from_dict(raw["mlp"], where + "mlp.")
-            else:
-                source = int(source)
-                if not 0 <= source < i:
-                    raise ConfigError(f"config.json: {where}weights_of must name an earlier layer")
-                if layers[source].weights_of is not None:  # a layer that borrows in turn: its owner
-                    source = layers[source].weights_of
-                # the tensors are the owner's, so the owner's sizes are the ones that count
-                kind, mixer, mlp = layers[source].type, layers[source].mixer, layers[source].mlp
-            layers.append(TazunexLayerConfig(kind, mixer, mlp, source))
+            mixer = _MIXERS[kind].from_dict(_mapping(raw, "mixer", where), where + "mixer.")
+            mlp = None if raw.get("mlp") is None else DenseFeedForwardConfig.from_dict(raw["mlp"], where + "mlp.")
+            slots[i] = TazunexLayerConfig(kind, mixer, mlp, None)
+        for i, raw in enumerate(raw_layers):  # the layers that borrow them, before or behind their owner
+            if raw.get("weights_of") is None:
+                continue
+            where = f"layers[{i}]."
+            source, seen = int(raw["weights_of"]), {i}
+            while 0 <= source < len(raw_layers) and raw_layers[source].get("weights_of") is not None:
+                if source in seen:
+                    break
+                seen.add(source)
+                source = int(raw_layers[source]["weights_of"])  # a layer that borrows in turn: its owner
+            owner = slots[source] if 0 <= source < len(raw_layers) and source not in seen else None
+            if owner is None or owner.weights_of is not None:
+                raise ConfigError(f"config.json: {where}weights_of must name a layer that has tensors of its own")
+            # the tensors are the owner's, so the owner's sizes are the ones that count
+            slots[i] = TazunexLayerConfig(owner.type, owner.mixer, owner.mlp, source)
+        layers = [layer for layer in slots if layer is not None]
+        assert len(layers) == len(raw_layers)
         cap = d.get("logit_softcap")
         cap = 0.0 if cap is None else float(cap)
         if cap < 0:

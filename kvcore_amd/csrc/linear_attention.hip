@@ -417,7 +417,8 @@ __global__ __launch_bounds__(256) void max_gates_kernel(
   float* ms = m_state + static_cast<int64_t>(slots[r]) * nh + h;
   float m = positions[b] == 0 ? 0.f : *ms;
   float mine = m;
-  for (int l = 0; l < kWave; ++l) {
+  const int runs = (n + run - 1) / run;  // lanes whose run holds a token: one for a single token
+  for (int l = 0; l < runs; ++l) {
     if (l == lane) mine = m;
     m = fmaxf(m + __shfl(A, l, kWave), __shfl(B, l, kWave));
   }

@@ -51,10 +51,8 @@ def tazunex_spec(config: TazunexConfig) -> ModelSpec:
 
     layers: list[LayerSpec] = []
     spec_index: dict[int, int] = {}  # config layer -> index among the layers that own tensors
-    schedule: list[ScheduleEntry] = []
     for i, layer in enumerate(config.layers):
         if layer.weights_of is not None:
-            schedule.append(ScheduleEntry(spec_index[layer.weights_of]))
             continue
         m = layer.mixer
         position = None
@@ -91,11 +89,13 @@ def tazunex_spec(config: TazunexConfig) -> ModelSpec:
                 "float32_result": True})
             norms = {"norm1": norm(), "norm1b": norm(), "norm2": norm(), "norm2b": norm()}
         spec_index[i] = len(layers)
-        schedule.append(ScheduleEntry(len(layers)))
         layers.append(LayerSpec(
             prefix=f"l{i}", mixer=mixer, ffn=ffn, norms=norms, position=position,
             block=PartSpec("sandwich_norm", {"mixer_name": "mix", "ffn_name": "mlp"})))
 
+    # a layer that borrows names its owner again, whichever of the two comes first
+    schedule = [ScheduleEntry(spec_index[i if layer.weights_of is None else layer.weights_of])
+                for i, layer in enumerate(config.layers)]
     return ModelSpec(
         vocab_size=config.vocab, hidden_size=H, max_position_embeddings=config.max_position_embeddings,
         layers=tuple(layers), final_norm=norm(), positions=tuple(positions), schedule=tuple(schedule),

@@ -49,6 +49,21 @@ def test_a_layer_that_borrows_tensors_is_a_second_run_of_its_owner():
     assert shapes == [(3, 24, 41), (3,), (3, 24, 41), (3,)]
 
 
+def test_an_owner_may_stand_behind_the_layer_that_borrows_from_it():
+    import copy
+
+    config = copy.deepcopy(CONFIG_A)
+    order = [3, 4, 0, 1, 2]  # the borrowed runs first
+    layers = [copy.deepcopy(config["layers"][i]) for i in order]
+    for layer in layers:
+        if "weights_of" in layer:
+            layer["weights_of"] = order.index(layer["weights_of"])
+    config["layers"] = layers
+    spec = spec_of(config)
+    assert [l.prefix for l in spec.layers] == ["l2", "l3", "l4"]
+    assert [e.layer for e in spec.resolved_schedule()] == [0, 1, 0, 1, 2]
+
+
 def test_rotations_are_shared_by_layers_with_the_same_constants():
     spec = spec_of(CONFIG_B)
     kinds = [(p.args["rot_dim"], p.args["theta"], p.args["interleaved"]) for p in spec.positions]
