@@ -346,10 +346,12 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
 // residual[t, :] += post_gain * delta[t, :] / sqrt(mean(delta[t, :]^2) + eps), and then, if out is
 // not null, out[t, :] = next_gain * residual[t, :] / sqrt(mean(residual[t, :]^2) + next_eps): the norm
 // behind a sublayer, the sum into the float32 stream and the norm before the next sublayer in one
-// pass.  delta is float32 (delta_dtype 0) or bfloat16 (1); out likewise (out_dtype).
+// pass.  delta is float32 (delta_dtype 0) or bfloat16 (1); out likewise (out_dtype).  slices > 1:
+// delta holds [slices, T, H] float32 partial sums of a product cut along K (kvc_gemm_mid_bf16 mode
+// 2) and a row of the result is their sum in slice order.
 int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* delta, int delta_dtype,
                       const float* post_gain, float eps, const float* next_gain, float next_eps,
-                      int T, int H, kvc_stream stream);
+                      int T, int H, int slices, kvc_stream stream);
 // Rows of qkv are [nq | nk | ...]: the first nq values (all query heads at once) are divided by
 // their root mean square (eps inside the root) and multiplied by q_gain [nq], the next nk values
 // likewise with k_gain [nk], in place; with copy_k the nk values as they were before the norm

@@ -48,24 +48,44 @@ __device__ __forceinline__ void st8(bf16_t* p, const float* v) {
   *reinterpret_cast<uint4*>(p) = a;
 }
 
+// A chunk of 8 values of a sublayer's result: the value itself, or, where the product before left
+// partial sums of slices along K ([slices, T, H] float32), their sum in slice order.
+template <typename TD>
+__device__ __forceinline__ void ld8_sum(const TD* p, int slices, int64_t slice_stride, float* v) {
+  ld8(p, v);
+  for (int s = 1; s < slices; ++s) {
+    float u[8];
+    ld8(p + s * slice_stride, u);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] += u[i];
+  }
+}
+template <typename TD>
+__device__ __forceinline__ float ld_sum(const TD* p, int slices, int64_t slice_stride) {
+  float v = to_float(p[0]);
+  for (int s = 1; s < slices; ++s) v += to_float(p[s * slice_stride]);
+  return v;
+}
+
 // Any width: three passes over memory, each thread rereading what it wrote itself.
 template <typename TD, typename TO>
 __global__ __launch_bounds__(256) void norm_add_norm_kernel(
     TO* __restrict__ out, float* __restrict__ residual, const TD* __restrict__ delta,
-    const float* __restrict__ post_gain, float eps, const float* __restrict__ next_gain, float next_eps, int H) {
+    const float* __restrict__ post_gain, float eps, const float* __restrict__ next_gain, float next_eps, int H,
+    int slices, int64_t slice_stride) {
   __shared__ float scratch[16];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
   float* r = residual + base;
   const TD* dl = delta + base;
   float sd = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float v = to_float(dl[i]);
+    const float v = ld_sum(dl + i, slices, slice_stride);
     sd += v * v;
   }
   const float inv_d = rsqrtf(block_sum(sd, scratch) / static_cast<float>(H) + eps);
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    const float v = r[i] + post_gain[i] * (to_float(dl[i]) * inv_d);
+    const float v = r[i] + post_gain[i] * (ld_sum(dl + i, slices, slice_stride) * inv_d);
     r[i] = v;
     ss += v * v;
   }
@@ -80,7 +100,8 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(
 template <typename TD, typename TO, int NCH>
 __global__ __launch_bounds__(256) void norm_add_norm_vec_kernel(
     TO* __restrict__ out, float* __restrict__ residual, const TD* __restrict__ delta,
-    const float* __restrict__ post_gain, float eps, const float* __restrict__ next_gain, float next_eps, int H) {
+    const float* __restrict__ post_gain, float eps, const float* __restrict__ next_gain, float next_eps, int H,
+    int slices, int64_t slice_stride) {
   __shared__ float scratch[16];
   const int64_t base = static_cast<int64_t>(blockIdx.x) * H;
   float d[NCH][8], v[NCH][8];
@@ -89,7 +110,7 @@ __global__ __launch_bounds__(256) void norm_add_norm_vec_kernel(
   for (int c = 0; c < NCH; ++c) {
     const int e = (c * 256 + threadIdx.x) * 8;
     if (e < H) {
-      ld8(delta + base + e, d[c]);
+      ld8_sum(delta + base + e, slices, slice_stride, d[c]);
       ld8(residual + base + e, v[c]);
 #pragma unroll
       for (int i = 0; i < 8; ++i) sd += d[c][i] * d[c][i];
@@ -128,7 +149,8 @@ __global__ __launch_bounds__(256) void norm_add_norm_vec_kernel(
 
 template <typename TD, typename TO>
 void launch_norm_add_norm(TO* out, float* residual, const TD* delta, const float* post_gain, float eps,
-                          const float* next_gain, float next_eps, int T, int H, hipStream_t stream) {
+                          const float* next_gain, float next_eps, int T, int H, int slices, hipStream_t stream) {
+  const int64_t slice_stride = static_cast<int64_t>(T) * H;
   const auto misaligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) != 0; };
   const bool vec = H % 8 == 0 && H <= 8 * 2048 && !misaligned(out) && !misaligned(residual) && !misaligned(delta) &&
                    !misaligned(post_gain) && !misaligned(next_gain);
@@ -136,7 +158,7 @@ void launch_norm_add_norm(TO* out, float* residual, const TD* delta, const float
     const int nch = (H + 2047) / 2048;
 #define KVC_NAN_CASE(NN)                                                                                   \
   hipLaunchKernelGGL((norm_add_norm_vec_kernel<TD, TO, NN>), dim3(T), dim3(256), 0, stream, out, residual, \
-                     delta, post_gain, eps, next_gain, next_eps, H)
+                     delta, post_gain, eps, next_gain, next_eps, H, slices, slice_stride)
     if (nch <= 1) KVC_NAN_CASE(1);
     else if (nch <= 2) KVC_NAN_CASE(2);
     else if (nch <= 4) KVC_NAN_CASE(4);
@@ -145,7 +167,7 @@ void launch_norm_add_norm(TO* out, float* residual, const TD* delta, const float
     return;
   }
   hipLaunchKernelGGL((norm_add_norm_kernel<TD, TO>), dim3(T), dim3(256), 0, stream, out, residual, delta,
-                     post_gain, eps, next_gain, next_eps, H);
+                     post_gain, eps, next_gain, next_eps, H, slices, slice_stride);
 }
 
 // One block a token.  The sums of squares of the two sections first (the raw keys copied behind
@@ -235,15 +257,16 @@ __global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ out, con
 
 extern "C" int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* delta, int delta_dtype,
                                  const float* post_gain, float eps, const float* next_gain, float next_eps,
-                                 int T, int H, kvc_stream stream) {
-  if (T < 0 || H <= 0) return kvc_fail("kvc_norm_add_norm: bad sizes");
+                                 int T, int H, int slices, kvc_stream stream) {
+  if (T < 0 || H <= 0 || slices < 1) return kvc_fail("kvc_norm_add_norm: bad sizes");
+  if (slices > 1 && delta_dtype != 0) return kvc_fail("kvc_norm_add_norm: partial sums are float32");
   if (residual == nullptr || delta == nullptr || post_gain == nullptr) return kvc_fail("kvc_norm_add_norm: null operand");
   if (out != nullptr && next_gain == nullptr) return kvc_fail("kvc_norm_add_norm: the second norm needs its gain");
   if (T == 0) return 0;
   if (out == nullptr) next_gain = post_gain;  // never read
 #define KVC_NAN(TD, TO)                                                                                         \
   launch_norm_add_norm<TD, TO>(static_cast<TO*>(out), residual, static_cast<const TD*>(delta), post_gain, eps, \
-                               next_gain, next_eps, T, H, S(stream))
+                               next_gain, next_eps, T, H, slices, S(stream))
   if (delta_dtype == 0 && out_dtype == 0) {
     KVC_NAN(float, float);
   } else if (delta_dtype == 0 && out_dtype == 1) {

@@ -43,7 +43,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_residual_add2": [P, P, I, P, I, I, I, P],
         "kvc_silu_mul": [P, P, I, I, I, P],
         "kvc_gate_mul": [P, P, I, I, I, I, P],
-        "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, P],
+        "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, I, P],
         "kvc_wide_qk_norm": [P, L, P, P, F, I, I, I, I, I, P],
         "kvc_head_gate": [P, P, L, P, L, I, I, I, I, I, I, P],
         "kvc_latent_rows": [P, L, P, P, L, P, L, P, P, F, I, I, I, I, I, P],
@@ -774,6 +774,27 @@ class NormedRows:
     data: torch.Tensor
 
 
+@dataclass
+class SliceSink:
+    """Where the last product of a part goes when the block behind it norms the result before
+    it joins the stream (steps of 17 to 192 rows): ``slices`` is float32 room for the partial
+    sums of a product cut along K (``mid_slices_bound(N) * T * N`` values).  ``linear`` leaves
+    them there and returns :class:`SlicedRows`; ``norm_add_norm`` sums them on its way."""
+
+    slices: torch.Tensor
+
+
+@dataclass
+class SlicedRows:
+    """``count`` partial sums ``[count, T, N]`` float32 at the start of ``data``'s storage: rows
+    of a product that the consumer adds up (one slice is the product itself)."""
+
+    data: torch.Tensor
+    count: int
+    rows: int
+    width: int
+
+
 # The most rows the kernel that shares its rows through LDS takes (twelve tiles of 16 a wave).
 # Measured on the 8B shape against the vendor's products with a norm kernel between them, a
 # whole decode step: 72 rows 5.93 against 6.66 ms, 96 rows 6.53 against 7.72, 128 rows 7.57
@@ -983,6 +1004,27 @@ def _sink_mid(sink: ResidualSink, x: torch.Tensor, w: torch.Tensor, bias: torch.
     return NormedRows(sink.out)
 
 
+def _slices_mid(sink: SliceSink, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None) -> SlicedRows:
+    """A product of 17 to 192 rows whose float32 sums a norm consumes: partial sums of slices
+    along K where the weight-streaming kernel takes the shape (as ``_sink_mid`` decides), else
+    the unrounded product itself as the one slice."""
+    M, K = x.shape
+    N = w.shape[0]
+    if sink.slices.dtype != torch.float32 or not sink.slices.is_contiguous():
+        raise KernelError("linear: the room for partial sums must be contiguous float32")
+    ours = (N < 8192 or K > 8192) and mid_rows_ok(M, bool(_streamed(w, N)[1]), MID_ROWS) and bias is None
+    if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and mid_operands_ok(x, w) and N % 8 == 0:
+        slices = mid_slices(N, K)
+        if sink.slices.numel() < slices * M * N:
+            raise KernelError("linear: the room for partial sums is too small")
+        gemm_mid(None, x, w, mode=2, partial=sink.slices)
+        return SlicedRows(sink.slices, slices, M, N)
+    if sink.slices.numel() < M * N:
+        raise KernelError("linear: the room for partial sums is too small")
+    linear(sink.slices.view(-1)[: M * N].view(M, N), x, w, bias)
+    return SlicedRows(sink.slices, 1, M, N)
+
+
 def linear_silu_mul(out: torch.Tensor, x: torch.Tensor | ScaledRows, w: torch.Tensor,
                     bias: torch.Tensor | None, scratch, act: str = "silu") -> None:
     """``out = act(x @ wg.T) * (x @ wu.T)`` with ``wg`` the first half of ``w``'s rows and
@@ -1031,6 +1073,10 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
     (few rows of bfloat16 only) the norm before or after the product is folded into it; a
     sink returns the :class:`ScaledRows` it made, or, in a step of 17 to 192 rows, where it
     finishes the norm itself, :class:`NormedRows`."""
+    if isinstance(out, SliceSink):
+        if isinstance(x, ScaledRows):
+            raise KernelError("linear: a product that leaves partial sums takes plain rows")
+        return _slices_mid(out, x, w, bias)
     if isinstance(out, ResidualSink) and out.slices is not None:
         if isinstance(x, ScaledRows):
             raise KernelError("linear: a sink that finishes the norm itself takes plain rows")
@@ -1421,15 +1467,23 @@ def max_gated_finish(out: torch.Tensor, o: torch.Tensor, m: torch.Tensor, gate: 
         "kvc_max_gated_finish")
 
 
-def norm_add_norm(out: torch.Tensor | None, residual: torch.Tensor, delta: torch.Tensor,
+def norm_add_norm(out: torch.Tensor | None, residual: torch.Tensor, delta: "torch.Tensor | SlicedRows",
                   post_gain: torch.Tensor, eps: float, next_gain: torch.Tensor | None = None,
                   next_eps: float | None = None) -> None:
     """``residual += post_gain * delta / rms(delta)``, then, given ``out``, ``out = next_gain *
     residual / rms(residual)``: the norm behind a sublayer, the sum into the float32 stream and the
     norm before the next sublayer in one pass (both roots hold their eps).  ``delta`` is float32
-    or bfloat16."""
+    or bfloat16, or the :class:`SlicedRows` that a product left (their sum is the result)."""
     T, H = residual.shape
-    if delta.shape != (T, H) or not delta.is_contiguous() or not residual.is_contiguous() or post_gain.shape != (H,):
+    slices = 1
+    if isinstance(delta, SlicedRows):
+        if (delta.rows, delta.width) != (T, H) or delta.data.dtype != torch.float32 \
+                or delta.data.numel() < delta.count * T * H or not delta.data.is_contiguous():
+            raise KernelError("norm_add_norm: the partial sums do not fit")
+        slices, delta = delta.count, delta.data
+    elif delta.shape != (T, H) or not delta.is_contiguous():
+        raise KernelError("norm_add_norm: shapes do not match")
+    if not residual.is_contiguous() or post_gain.shape != (H,):
         raise KernelError("norm_add_norm: shapes do not match")
     if out is not None and (out.shape != (T, H) or not out.is_contiguous() or next_gain is None
                             or next_gain.shape != (H,)):
@@ -1439,7 +1493,7 @@ def norm_add_norm(out: torch.Tensor | None, residual: torch.Tensor, delta: torch
         _dev(residual, "residual", torch.float32), _dev(delta, "delta"), _code(delta, "delta"),
         _dev(post_gain, "post_gain", torch.float32), float(eps),
         None if out is None else _dev(next_gain, "next_gain", torch.float32),
-        float(eps if next_eps is None else next_eps), T, H, _stream()), "kvc_norm_add_norm")
+        float(eps if next_eps is None else next_eps), T, H, slices, _stream()), "kvc_norm_add_norm")
 
 
 def wide_qk_norm(qkv: torch.Tensor, q_gain: torch.Tensor, k_gain: torch.Tensor, eps: float, *,

@@ -104,6 +104,10 @@ class PagedAttention(Mixer):
     def takes_sink(self) -> bool:  # the output product's rows are whole heads
         return self.o_size % 8 == 0 and not self.float32_result
 
+    @property
+    def takes_slice_sink(self) -> bool:  # float32 partial sums whatever the result's type
+        return self.o_size % 8 == 0
+
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, bias: bool = False, window: int = 0, page_size: int | None = None,
                  v_head_dim: int | None = None, qk_norm_eps: float | None = None,

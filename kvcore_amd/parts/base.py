@@ -276,10 +276,11 @@ class StreamOp(Part):
 
 
 class FeedForward(Part):
-    """``takes_scaled_rows`` and ``takes_sink`` as for :class:`Mixer`."""
+    """``takes_scaled_rows``, ``takes_sink`` and ``takes_slice_sink`` as for :class:`Mixer`."""
 
     takes_scaled_rows = False
     takes_sink = False
+    takes_slice_sink = False
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", call: "LayerCall") -> torch.Tensor:
         raise NotImplementedError

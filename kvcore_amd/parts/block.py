@@ -179,7 +179,8 @@ class SandwichNormBlock(Block):
 
     def _join(self, result, residual, ctx, post, following, name: str):
         """``residual += post(result)``, and the rows of the norm ``following`` (a (gain, eps) or
-        None) into the step buffer ``name``."""
+        None) into the step buffer ``name``.  ``result`` is a tensor or the partial sums that a
+        part's last product left (``ops.SlicedRows``)."""
         post_gain, post_eps = post
         if following is None:
             ops.norm_add_norm(None, residual, result, post_gain, post_eps)
@@ -187,6 +188,16 @@ class SandwichNormBlock(Block):
         rows = ctx.buf(name, residual.shape[1])
         ops.norm_add_norm(rows, residual, result, post_gain, post_eps, following[0], following[1])
         return rows
+
+    def _slice_sink(self, part, residual, ctx):
+        """In a step of a few dozen rows a part's last product may leave partial sums of slices
+        along K, which the norm behind it adds up on its way: the ``ops.SliceSink`` for that, or
+        None where the step or the part does not take one."""
+        H = residual.shape[1]
+        if not (getattr(part, "takes_slice_sink", False) and H % 8 == 0
+                and ops.rows_sinkable(ctx.num_tokens, ctx.dtype)):
+            return None
+        return ops.SliceSink(ctx.buffers.get("block_slices", ops.mid_slices_bound(H) * ops.MID_ROWS, H, torch.float32))
 
     def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
         if isinstance(delta, ops.ScaledRows):
@@ -197,16 +208,17 @@ class SandwichNormBlock(Block):
             x = ctx.buf("block_x", residual.shape[1])
             self.norms[self.norm_names[0]].forward_fused(x, residual, delta)
         following = next_block.input_gain(scaled=False) if next_block is not None else None
-        a = self.mixer.forward(x, ctx, call)
+        sink = self._slice_sink(self.mixer, residual, ctx)
+        a = self.mixer.forward(x, ctx, call) if sink is None else self.mixer.forward(x, ctx, call, sink=sink)
         if self.mixer_only:
             rows = self._join(a, residual, ctx, self._gain(1), following, "block_x")
             return None if rows is None else ops.NormedRows(rows)
         x2 = self._join(a, residual, ctx, self._gain(1), self._gain(2), "block_x2")
-        f = self.ffn.forward(x2, ctx, call)
+        sink = self._slice_sink(self.ffn, residual, ctx)
+        f = self.ffn.forward(x2, ctx, call) if sink is None else self.ffn.forward(x2, ctx, call, sink=sink)
         rows = self._join(f, residual, ctx, self._gain(3), following, "block_x")
         return None if rows is None else ops.NormedRows(rows)
 
 
-register_block("prenorm", PreNormBlock)
 register_block("sandwich_norm", SandwichNormBlock)
 register_block("parallel_residual", ParallelResidualBlock)

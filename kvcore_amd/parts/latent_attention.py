@@ -36,6 +36,10 @@ class LatentAttention(PagedAttention):
     takes_scaled_rows = False  # the input feeds the gate as well
     takes_sink = False
 
+    @property
+    def takes_slice_sink(self) -> bool:
+        return (self.heads * self.kv_rank) % 8 == 0
+
     def __init__(self, *, hidden_size: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
                  q_rank: int, scale: float, eps: float, window: int = 0, page_size: int | None = None,
                  gated: bool = True, tensor_names: dict[str, str] | None = None,
@@ -128,6 +132,8 @@ class LatentAttention(PagedAttention):
             kept.view(-1, nh, rank).copy_(attn.view(-1, nh, self.row)[:, :, self.rot:])
         else:
             kept = attn
+        if sink is not None:
+            return ops.linear(sink, kept, p["o_latent.weight"])
         if self.float32_result:
             out = ctx.buf("mixer_out_f32", self.hidden_size, torch.float32)
         else:

@@ -236,6 +236,10 @@ class MaxGatedMatrixMemory(_MatrixStateMixer):
     def product_weights(self) -> tuple[str, ...]:
         return ("in_proj.weight", "o.weight")
 
+    @property
+    def takes_slice_sink(self) -> bool:
+        return self.inner % 8 == 0
+
     def state_needs(self) -> tuple[StateNeed, ...]:
         # the matrices with the normaliser as their last column, and the running maxima
         return (StateNeed((self.heads, ops.linear_state_rows(self.dim), self.vdim + 1)), StateNeed((self.heads,)))
@@ -261,6 +265,8 @@ class MaxGatedMatrixMemory(_MatrixStateMixer):
         normed = ctx.buf(f"ms_normed:{inner}", inner)
         ops.max_gated_finish(normed, o, m, proj[:, 2 * qk + inner:2 * qk + 2 * inner], p["norm"], self.eps,
                              self.den_eps, nh, self.vdim)
+        if sink is not None:
+            return ops.linear(sink, normed, p["o.weight"])
         if self.float32_result:
             out = ctx.buf("mixer_out_f32", self.hidden_size, torch.float32)
         else:

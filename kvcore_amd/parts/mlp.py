@@ -23,6 +23,10 @@ class SwiGLU(FeedForward):
     def takes_sink(self) -> bool:
         return self.intermediate_size % 8 == 0 and not self.float32_result
 
+    @property
+    def takes_slice_sink(self) -> bool:  # float32 partial sums whatever the result's type
+        return self.intermediate_size % 8 == 0
+
     def __init__(self, *, hidden_size: int, intermediate_size: int, bias: bool = False,
                  gate_name: str = "gate_proj", up_name: str = "up_proj", down_name: str = "down_proj",
                  suffix: str = ".weight", sized_buffers: bool = False, activation: str = "silu",

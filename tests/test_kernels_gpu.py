@@ -1075,15 +1075,15 @@ def test_decode_attention_says_what_it_does_not_serve(ops):
 def test_paged_attention_refuses_unsupported_head_sizes(ops):
     from kvcore_amd.ops.library import KernelError
 
-    kc, vc = make_cache(2, 1, 4, 272, torch.float32)
-    q = rnd(1, 272)
-    with pytest.raises(KernelError, match="at most 256"):
-        ops.paged_attention(torch.empty(1, 272, device=DEV), q, kc, vc,
+    kc, vc = make_cache(2, 1, 4, 528, torch.float32)
+    q = rnd(1, 528)
+    with pytest.raises(KernelError, match="at most 512"):
+        ops.paged_attention(torch.empty(1, 528, device=DEV), q, kc, vc,
                             table=torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                             positions=torch.zeros(1, dtype=torch.int32, device=DEV),
                             token_req=torch.zeros(1, dtype=torch.int32, device=DEV),
                             slots=torch.zeros(1, dtype=torch.int32, device=DEV),
-                            nh=1, nkv=1, d=272, scale=1.0)
+                            nh=1, nkv=1, d=528, scale=1.0)
 
 
 def test_table_update(ops):

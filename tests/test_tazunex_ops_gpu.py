@@ -48,6 +48,53 @@ def test_norm_behind_a_sublayer_sum_and_next_norm(H, delta_dtype):
     assert rel(res, want_r) < 1e-6
 
 
+@pytest.mark.parametrize("H,slices", [(96, 3), (100, 2), (2048, 4)])
+def test_norm_behind_a_sublayer_adds_up_partial_sums(H, slices):
+    """The result of the sublayer as partial sums of slices, as a product cut along K leaves them."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(H + slices)
+    T, eps = 29, 1e-5
+    r = torch.randn(T, H, generator=gen, dtype=F64)
+    parts = torch.randn(slices, T, H, generator=gen, dtype=F64).float().double()
+    g1, g2 = 1 + 0.3 * torch.randn(H, generator=gen, dtype=F64), 1 + 0.3 * torch.randn(H, generator=gen, dtype=F64)
+    want_r = r + plain.rms(parts.sum(0), eps) * g1
+    want_x = plain.rms(want_r, eps) * g2
+    room = torch.full((slices * T * H + 64,), float("nan"), device=DEV)
+    room[: slices * T * H] = gpu(parts).view(-1)
+    res, out = gpu(r), torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.norm_add_norm(out, res, ops.SlicedRows(room, slices, T, H), gpu(g1), eps, gpu(g2), eps)
+    assert rel(res, want_r) < 1e-6 and rel(out, want_x) < 4e-3
+
+
+@pytest.mark.parametrize("M,N,K,packed", [(40, 1024, 2048, True), (64, 512, 4096, True), (40, 1024, 2048, False),
+                                          (23, 96, 80, False), (100, 2048, 8192, True)])
+def test_a_product_that_leaves_partial_sums_for_the_norm_behind_it(M, N, K, packed):
+    """``linear`` into a ``SliceSink`` and the norm that adds the slices up, against the plain
+    product and norm on the same rounded operands: shapes that the weight-streaming kernel cuts
+    along K, and shapes it does not take (then the one slice is the product itself)."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).to(torch.bfloat16)
+    r = torch.randn(M, N, generator=gen, dtype=F64)
+    g1 = 1 + 0.3 * torch.randn(N, generator=gen, dtype=F64)
+    eps = 1e-6
+    want_r = r + plain.rms(x.double() @ w.double().T, eps) * g1
+    wd = gpu(w, torch.bfloat16)
+    if packed:
+        ops.pack_weight(wd)
+    room = torch.full((ops.mid_slices_bound(N) * ops.MID_ROWS * N,), float("nan"), device=DEV)
+    got = ops.linear(ops.SliceSink(room), gpu(x, torch.bfloat16), wd)
+    assert isinstance(got, ops.SlicedRows) and (got.rows, got.width) == (M, N)
+    if packed and K % 512 == 0:
+        assert got.count == ops.mid_slices(N, K)
+    res = gpu(r)
+    ops.norm_add_norm(None, res, got, gpu(g1), eps)
+    assert rel(res, want_r) < 1e-5
+
+
 @pytest.mark.parametrize("nq,nk,extra", [(128, 64, 0), (16, 16, 5), (3, 1, 0), (4096, 1024, 8)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_norm_over_a_whole_projection(nq, nk, extra, dtype):
@@ -393,7 +440,7 @@ def test_a_sink_that_outweighs_every_key():
 
 
 @pytest.mark.parametrize("kernel,nsplit", [("portion", 1), ("portion", 3), ("single", 1), ("single", 4)])
-@pytest.mark.parametrize("H,G,d,window", [(8, 2, 64, 48), (4, 4, 128, 0), (4, 1, 128, 100), (16, 2, 64, 1), (6, 1, 96, 136)])
+@pytest.mark.parametrize("H,G,d,window", [(8, 2, 64, 48), (4, 4, 128, 0), (4, 1, 128, 100), (16, 2, 64, 1), (6, 1, 96, 150)])
 def test_matrix_core_kernels_with_windows_and_sinks(kernel, nsplit, H, G, d, window):
     """The bfloat16 kernels for portions and for single tokens against the plain function on the
     same rounded values: every position of a prompt of 300 tokens (windows that are no multiple of
