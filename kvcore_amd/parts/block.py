@@ -220,5 +220,6 @@ class SandwichNormBlock(Block):
         return None if rows is None else ops.NormedRows(rows)
 
 
+register_block("prenorm", PreNormBlock)
 register_block("sandwich_norm", SandwichNormBlock)
 register_block("parallel_residual", ParallelResidualBlock)
