@@ -11,7 +11,7 @@
 // only: not on the batch it is in nor on how its request was cut into steps.  Two options:
 // `slopes` (a value per query head) takes slope * (position - key position) off every score, and
 // `chunk` lets a token see only the keys of its own chunk of that many positions; `sinks` (a value
-// per query head) adds exp(sink) to the softmax's denominator, a score that has no key or value.
+// per query head) adds exp(sink) to the softmax's denominator and nothing to the weighted sum.
 
 #include <hip/hip_runtime.h>
 
@@ -82,8 +82,8 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
   for (int i = lane; i < d; i += kWave) q_s[wave][i] = to_float(qh[i]);
   __syncthreads();
 
-  // a sink is a score with no key and no value that the denominator counts once: the running
-  // softmax starts from it instead of from nothing
+  // a sink is one more logit in the denominator that brings no value along: the running softmax
+  // starts from it instead of from nothing
   float m = -INFINITY, l = 0.f;
   if (sinks != nullptr) {
     m = sinks[h];

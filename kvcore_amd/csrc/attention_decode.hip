@@ -71,7 +71,7 @@ struct DecodeArgs {
   int window;
   const float* slopes;  // [nh] or null: slope * (position - key position) comes off the score
   int chunk;            // > 0: only the keys of the token's own chunk of so many positions
-  const float* sinks;   // [nh] or null: exp(sink) joins the softmax's denominator, with no key or value
+  const float* sinks;   // [nh] or null: exp(sink) joins the softmax's denominator and brings no value along
   int nsplit;
   int lds_pages;  // page ids of a block's range that fit in LDS
 };

@@ -122,8 +122,8 @@ int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_
 // pages [kv head, page_size, d], V pages [kv head, dv, page_size]); out is [T, nh*dv].
 // slopes (float32 [nh], or null): slopes[h] * (p - key position) is taken off every score of head
 // h.  chunk > 0: a token sees only the keys j with j / chunk == p / chunk.  sinks (float32 [nh],
-// or null): exp(sinks[h]) is added to the softmax's denominator of head h, a score that has no
-// key and no value and is not scaled.
+// or null): exp(sinks[h]) is added to the softmax's denominator of head h: a logit of its own,
+// taken as it is (scale does not apply), that brings no value into the weighted sum.
 int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                         const void* v_cache, const int32_t* table, int table_stride,
                         const int32_t* positions, const int32_t* token_req,
