@@ -498,6 +498,48 @@ extern "C" int kvc_gate_mul(void* out, const void* gate_up, int T, int I, int ac
   return kvc_check_launch("kvc_gate_mul");
 }
 
+// ------------------------------------------------------------- activation without a gate
+// out = act(x) elementwise, in float32 from either storage type; act 0: the square of relu.
+template <typename T>
+__global__ void activation_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t n, int act) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const float v = fmaxf(to_float(x[idx]), 0.f);
+  out[idx] = from_float<T>(v * v);
+}
+
+template <typename T>
+__global__ void activation_vec_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t n8, int act) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n8) return;
+  float v[8];
+  load8(x + idx * 8, v);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float r = fmaxf(v[e], 0.f);
+    v[e] = r * r;
+  }
+  store8(out + idx * 8, v);
+}
+
+extern "C" int kvc_activation(void* out, const void* x, int64_t n, int act, int dtype, kvc_stream stream) {
+  if (n < 0) return kvc_fail("kvc_activation: bad size");
+  if (act != 0) return kvc_fail("kvc_activation: unknown activation");
+  if (n == 0) return 0;
+  if (n % 8 == 0 && (reinterpret_cast<uintptr_t>(out) % 16) == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0) {
+    const unsigned vblocks = static_cast<unsigned>((n / 8 + 255) / 256);
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL(activation_vec_kernel<Tp>, dim3(vblocks), dim3(256), 0, S(stream),
+                                          static_cast<Tp*>(out), static_cast<const Tp*>(x), n / 8, act));
+    return kvc_check_launch("kvc_activation");
+  }
+  const unsigned blocks = static_cast<unsigned>((n + 255) / 256);
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(activation_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),
+                                        static_cast<Tp*>(out), static_cast<const Tp*>(x), n, act));
+  return kvc_check_launch("kvc_activation");
+}
+
 // ----------------------------------------------------------------------- row gather
 template <typename TI, typename TO>
 __global__ void gather_rows_kernel(TO* __restrict__ out, const TI* __restrict__ in,

@@ -86,6 +86,9 @@ int kvc_silu_mul(void* out, const void* gate_up, int T, int I, int dtype, kvc_st
 // 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
 int kvc_gate_mul(void* out, const void* gate_up, int T, int I, int act, int dtype, kvc_stream stream);
 
+// out = act(x) elementwise over n values (in place is fine); act 0: the square of relu.
+int kvc_activation(void* out, const void* x, int64_t n, int act, int dtype, kvc_stream stream);
+
 // out[s, :] = in[rows[s], :]; `in` may be float32 (in_dtype 0) while out is dt.
 int kvc_gather_rows(void* out, const void* in, const int32_t* rows, int S, int H, int in_dtype,
                     int out_dtype, kvc_stream stream);
@@ -266,22 +269,27 @@ int kvc_head_rmsnorm_gate(void* out, int out_dtype, const float* o, const void* 
 // x row sorted[i] / in_div (in_div 0: row i itself) and writes out row i (out_sorted) or
 // sorted[i].  dtype is that of x and w.  packed: w is the copy kvc_pack_weight makes of the whole
 // stacked matrix (bfloat16, N a multiple of 16, K of 64).
+// score_fn 0: softmax over the experts, 1: sigmoid of each logit.  correction [E] (or null) is added
+// to the scores for the choice alone.  group_best 1 or 2: a group is worth its best choice score, or
+// the sum of its best two.  The weights are multiplied by weight_scale.
 int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
-                  int groups, int keep, kvc_stream stream);
+                  int groups, int keep, int score_fn, const float* correction, int group_best,
+                  float weight_scale, kvc_stream stream);
 // Tiles hold up to tile_rows rows, 16 or 64 (kvc_moe_tile_rows says which a step's size asks
 // for; 64 is for bfloat16 with K a multiple of 32).
 int kvc_moe_tile_rows(int pairs, int E);
 // The router's logits (x [T, H] of x_dtype times router [E, H] float32, float32 sums in one fixed order)
 // and the choice of kvc_moe_route in one kernel.
 int kvc_moe_router(int32_t* choice, float* weight, const void* x, int64_t x_stride, int x_dtype,
-                   const float* router, int T, int H, int E, int top, int groups, int keep, kvc_stream stream);
+                   const float* router, int T, int H, int E, int top, int groups, int keep, int score_fn,
+                   const float* correction, int group_best, float weight_scale, kvc_stream stream);
 int kvc_moe_max_tiles(int pairs, int E, int tile_rows);
 int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles, const int32_t* choice,
                   int pairs, int E, int max_tiles, int tile_rows, kvc_stream stream);
 int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                  const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
                  const int32_t* num_tiles, int max_tiles, int tile_rows, int N, int K, int in_div, int out_sorted,
-                 int gated, float limit, float alpha, int packed, kvc_stream stream);
+                 int gated, float limit, float alpha, float up_shift, int packed, kvc_stream stream);
 // out[t] = sum_c weight[t, c] * y[t * top + c] + add0[t] + add1[t] (either may be null; add0 of
 // dtype add0_dtype, add1 float32), float32.
 // accumulate: the sum is added into out instead of stored.
@@ -352,6 +360,10 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
 int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* delta, int delta_dtype,
                       const float* post_gain, float eps, const float* next_gain, float next_eps,
                       int T, int H, int slices, kvc_stream stream);
+// Rows of attn are [heads][2][dv]: out[t, h] = (a1 - lambda * a2) / sqrt(mean((a1 - lambda * a2)^2) + eps)
+// * post over the head's dv values, out [T, heads * dv]; float32 arithmetic.
+int kvc_diff_heads_norm(void* out, const void* attn, int64_t attn_stride, float lambda, float eps, float post,
+                        int T, int heads, int dv, int dtype, kvc_stream stream);
 // Rows of qkv are [nq | nk | ...]: the first nq values (all query heads at once) are divided by
 // their root mean square (eps inside the root) and multiplied by q_gain [nq], the next nk values
 // likewise with k_gain [nk], in place; with copy_k the nk values as they were before the norm
@@ -368,6 +380,16 @@ int kvc_latent_rows(void* cq, int64_t cq_stride, void* key, void* value, int64_t
 // e < n: a gate per head, and a run of each head's columns kept.  gate has the dtype of x and out.
 int kvc_head_gate(void* out, const void* x, int64_t x_stride, const void* gate, int64_t gate_stride,
                   int T, int heads, int head_stride, int skip, int n, int dtype, kvc_stream stream);
+
+// A residual stream of `copies` (1 to 8) rows a token, streams [T, copies, H] float32.  With y ([T, H]
+// of y_dtype): x_t <- sum_s mix[s * copies + t] x_s + mult * out_w[t] * y for all copies at once (mix
+// null: the identity, out_w null: ones).  Then, with out ([T, H] of out_dtype): u = sum_t in_w[t] x_t
+// (in_w null: ones), out = gain * u / sqrt(mean(u^2) + eps).
+int kvc_hyper_step(void* out, int out_dtype, float* streams, const void* y, int y_dtype, const float* mix,
+                   const float* out_w, float mult, const float* in_w, const float* gain, float eps, int T, int H,
+                   int copies, kvc_stream stream);
+// streams[t, c, :] = rows[t, :] for every copy c.
+int kvc_spread_streams(float* streams, const float* rows, int T, int H, int copies, kvc_stream stream);
 
 // C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) in float32 with float32 products and sums;
 // each element is one running sum over k = 0..K-1, whatever M is.

@@ -5,16 +5,19 @@
 // tokens x choices, tiles <= pairs / 16 + experts), so a step neither waits for the routing nor
 // changes its launches with it: a captured step replays for any routing.
 //
-//   kvc_moe_route    scores = softmax(logits) in float32; the `keep` groups whose best score is
-//                    highest; the `top` best experts of those groups (the lower index on a tie);
-//                    weights = chosen scores / (their sum + 1e-20).  A wave a token.
+//   kvc_moe_route    scores = softmax(logits) or sigmoid(logits) in float32; the choice is made on the
+//                    scores plus an optional correction per expert: the `keep` groups that are worth
+//                    most (a group's best choice score, or the sum of its best two); the `top` best
+//                    experts of those groups (the lower index on a tie); weights = the chosen experts'
+//                    plain scores / (their sum + 1e-20) * weight_scale.  A wave a token.
 //   kvc_moe_router   the router's product (float32 sums in one fixed order over rows of either dtype)
 //                    and the choice in one kernel.
 //   kvc_moe_align    pairs sorted by expert: sorted[i] = pair index (token * top + choice), and a
 //                    list of tiles of up to 16 (or 64) sorted rows that belong to one expert each.
 //   kvc_moe_gemm     for every tile, rows x that expert's matrix.  Gated: gate and up rows of the
 //                    expert side by side in one pass, and the activation
-//                    min(g, limit) * sigmoid(alpha * g) * (clamp(u, -limit, limit) + 1) on the way out.
+//                    min(g, limit) * sigmoid(alpha * g) * (clamp(u, -limit, limit) + up_shift) on the way
+//                    out (an infinite limit, alpha 1 and up_shift 0: silu(g) * u).
 //                    bfloat16 operands go through the matrix cores (16 x 16 x 32, the expert's rows as
 //                    the A operand, the tokens as B) with float32 sums; float32 operands, and rows
 //                    that 16-byte loads do not divide, are summed in float32 in index order.  A row's sums do not depend on which tile it is in.
@@ -37,10 +40,10 @@ namespace {
 constexpr int kTileRows = 16;
 constexpr int kBigTileRows = 64;
 
-__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha) {
+__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha, float shift) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
-  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  return g / (1.f + expf(-alpha * g)) * (u + shift);
 }
 
 // the lane that holds the largest value (the lowest index among equals) tells everyone
@@ -56,29 +59,55 @@ __device__ __forceinline__ void wave_argmax(float& val, int& idx) {
   }
 }
 
-// One token's choice by one wave: z [E] logits (global or LDS), sc [E] and gs [groups] LDS scratch
-// (sc may be z itself).
+// How a token's experts are chosen from its logits.  score_fn 0: softmax over the experts, 1: a
+// sigmoid of each logit.  The choice is made on score + correction[e] (correction may be null) and
+// may so be negative; the weights are the plain scores of the chosen, over their sum (+ 1e-20),
+// times weight_scale.  With keep < groups only the experts of the best `keep` of `groups` equal
+// groups of neighbours may be chosen; a group is worth the sum of its `group_best` (1 or 2) largest
+// choice scores.  The lower index wins a tie.
+struct RouteRule {
+  int top, groups, keep, score_fn, group_best;
+  const float* correction;
+  float weight_scale;
+};
+
+// One token's choice by one wave: z [E] logits (global or LDS), sc [E], pk [E] and gs [groups] LDS
+// scratch (sc may be z itself).
 __device__ __forceinline__ void route_one(int32_t* __restrict__ choice, float* __restrict__ weight, const float* z,
-                                          float* sc, float* gs, int lane, int E, int top, int groups, int keep) {
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += kWave) mx = fmaxf(mx, z[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += kWave) {
-    const float p = expf(z[e] - mx);
-    sc[e] = p;
-    sum += p;
+                                          float* sc, float* pk, float* gs, int lane, int E, const RouteRule& rule) {
+  const int top = rule.top, groups = rule.groups, keep = rule.keep;
+  if (rule.score_fn == 0) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += kWave) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += kWave) {
+      const float p = expf(z[e] - mx);
+      sc[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+    for (int e = lane; e < E; e += kWave) sc[e] *= inv;
+  } else {
+    for (int e = lane; e < E; e += kWave) sc[e] = 1.f / (1.f + expf(-z[e]));
   }
-  sum = wave_sum(sum);
-  const float inv = 1.f / sum;
-  for (int e = lane; e < E; e += kWave) sc[e] *= inv;
+  for (int e = lane; e < E; e += kWave) pk[e] = sc[e] + (rule.correction != nullptr ? rule.correction[e] : 0.f);
   __builtin_amdgcn_wave_barrier();
   const int per = E / groups;
   if (keep < groups) {
     for (int g = lane; g < groups; g += kWave) {
-      float best = -INFINITY;
-      for (int i = 0; i < per; ++i) best = fmaxf(best, sc[g * per + i]);
-      gs[g] = best;
+      float best = -INFINITY, second = -INFINITY;
+      for (int i = 0; i < per; ++i) {
+        const float s = pk[g * per + i];
+        if (s > best) {
+          second = best;
+          best = s;
+        } else if (s > second) {
+          second = s;
+        }
+      }
+      gs[g] = (rule.group_best >= 2 && per >= 2) ? best + second : best;
     }
     __builtin_amdgcn_wave_barrier();
     // the best `keep` groups are marked with +inf; the others' experts are taken out
@@ -97,7 +126,7 @@ __device__ __forceinline__ void route_one(int32_t* __restrict__ choice, float* _
       __builtin_amdgcn_wave_barrier();
     }
     for (int e = lane; e < E; e += kWave)
-      if (gs[e / per] != INFINITY) sc[e] = -1.f;  // scores are positive: never chosen before a kept one
+      if (gs[e / per] != INFINITY) pk[e] = -INFINITY;  // choice scores may be negative: minus infinity, not zero
     __builtin_amdgcn_wave_barrier();
   }
   float total = 0.f;
@@ -107,24 +136,26 @@ __device__ __forceinline__ void route_one(int32_t* __restrict__ choice, float* _
     float val = -INFINITY;
     int idx = 0x7fffffff;
     for (int e = lane; e < E; e += kWave) {
-      const float s = sc[e];
+      const float s = pk[e];
       if (s > val || (s == val && e < idx)) {
         val = s;
         idx = e;
       }
     }
     wave_argmax(val, idx);
-    if (idx >= E) { idx = 0; val = 0.f; }
-    if (val < 0.f) val = 0.f;  // fewer allowed experts than choices: a weight of zero
-    total += val;
+    if (idx >= E) idx = 0;
+    // fewer allowed experts than choices: a weight of zero
+    const float plain = (val == -INFINITY) ? 0.f : sc[idx];
+    total += plain;
     if (lane == c) {
-      mine = val;
+      mine = plain;
       mine_idx = idx;
     }
-    if (lane == 0) sc[idx] = -2.f;
+    __builtin_amdgcn_wave_barrier();
+    if (lane == 0) pk[idx] = -INFINITY;
     __builtin_amdgcn_wave_barrier();
   }
-  const float norm = 1.f / (total + 1e-20f);
+  const float norm = rule.weight_scale / (total + 1e-20f);
   if (lane < top) {
     choice[lane] = mine_idx;
     weight[lane] = mine * norm;
@@ -133,14 +164,14 @@ __device__ __forceinline__ void route_one(int32_t* __restrict__ choice, float* _
 
 __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
                                                         const float* __restrict__ logits, int T, int E,
-                                                        int top, int groups, int keep) {
+                                                        RouteRule rule) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  float* sc = lds + wave * (E + groups);  // scores, then the groups' best
+  float* sc = lds + wave * (2 * E + rule.groups);  // scores, choice scores, then the groups' worth
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;  // the whole wave
-  route_one(choice + static_cast<int64_t>(t) * top, weight + static_cast<int64_t>(t) * top,
-            logits + static_cast<int64_t>(t) * E, sc, sc + E, lane, E, top, groups, keep);
+  route_one(choice + static_cast<int64_t>(t) * rule.top, weight + static_cast<int64_t>(t) * rule.top,
+            logits + static_cast<int64_t>(t) * E, sc, sc + E, sc + 2 * E, lane, E, rule);
 }
 
 // The router whole: logits = x W^T in float32 (x of either dtype, its values as they are), then the
@@ -152,13 +183,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* __restrict__ ch
 template <typename T, int TOK>
 __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ choice, float* __restrict__ weight,
                                                          const T* __restrict__ x, int64_t x_stride,
-                                                         const float* __restrict__ wr, int T_, int H, int E, int top,
-                                                         int groups, int keep, int vectors) {
+                                                         const float* __restrict__ wr, int T_, int H, int E,
+                                                         RouteRule rule, int vectors) {
   constexpr int EB = 32, PR = EB + 1;
   extern __shared__ float lds[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   float* part = lds;                       // [256][EB + 1]
-  float* z = lds + 256 * PR;               // [TOK][E + groups]
+  float* z = lds + 256 * PR;               // [TOK][2 E + groups]
+  const int zrow = 2 * E + rule.groups;
   const int t0 = blockIdx.x * TOK;
   for (int e0 = 0; e0 < E; e0 += EB) {
     const int ne = (E - e0 < EB) ? E - e0 : EB;
@@ -205,7 +237,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ c
       if (threadIdx.x < ne) {
         float sum = 0.f;
         for (int l = 0; l < 256; ++l) sum += part[l * PR + threadIdx.x];
-        z[j * (E + groups) + e0 + threadIdx.x] = sum;
+        z[j * zrow + e0 + threadIdx.x] = sum;
       }
     }
   }
@@ -214,9 +246,9 @@ __global__ __launch_bounds__(256) void moe_router_kernel(int32_t* __restrict__ c
   for (int j = 0; j < TOK; ++j) {
     const int t = t0 + j;
     if (t >= T_) break;  // the whole wave
-    float* zr = z + j * (E + groups);
-    route_one(choice + static_cast<int64_t>(t) * top, weight + static_cast<int64_t>(t) * top, zr, zr, zr + E, lane, E,
-              top, groups, keep);
+    float* zr = z + j * zrow;
+    route_one(choice + static_cast<int64_t>(t) * rule.top, weight + static_cast<int64_t>(t) * rule.top, zr, zr, zr + E,
+              zr + 2 * E, lane, E, rule);
   }
 }
 
@@ -272,7 +304,7 @@ template <int GATED, typename TO, int PACKED>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
     const bf16_t* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
-    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
+    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha, float shift) {
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;
   const int e = tiles[3 * tile], r0 = tiles[3 * tile + 1], nr = tiles[3 * tile + 2];
@@ -362,7 +394,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   if (!row_ok) return;
   if (GATED) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] = clamped_glu(acc[i], acc2[i], limit, alpha);
+    for (int i = 0; i < 4; ++i) acc[i] = clamped_glu(acc[i], acc2[i], limit, alpha, shift);
   }
   const int64_t out_row = out_sorted ? r0 + li : pair;
   const int nf = n0 + 4 * lk;
@@ -378,7 +410,7 @@ template <int GATED, typename TO, int PACKED>
 __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
     TO* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ x, int64_t x_stride,
     const bf16_t* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
-    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
+    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha, float shift) {
   constexpr int NF = GATED ? 2 : 4;   // column blocks of 16 a wave
   constexpr int NR = kBigTileRows / 16;
   constexpr int KC = 64;              // values of K a pass (two matrix instructions deep)
@@ -484,7 +516,7 @@ __global__ __launch_bounds__(256) void moe_gemm_tiled_kernel(
       f32x4_t v = acc[f][r];
       if (GATED) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = clamped_glu(v[i], acc2[f][r][i], limit, alpha);
+        for (int i = 0; i < 4; ++i) v[i] = clamped_glu(v[i], acc2[f][r][i], limit, alpha, shift);
       }
       const int nf = n0 + 16 * f + 4 * lk;
       if (nf < N) store4<TO>(out + out_row * out_stride + nf, v, N - nf);
@@ -498,7 +530,7 @@ template <int GATED, typename TI, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     TO* __restrict__ out, int64_t out_stride, const TI* __restrict__ x, int64_t x_stride,
     const TI* __restrict__ w, const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles,
-    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha) {
+    const int32_t* __restrict__ num_tiles, int N, int K, int in_div, int out_sorted, float limit, float alpha, float shift) {
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;
   const int e = tiles[3 * tile], r0 = tiles[3 * tile + 1], nr = tiles[3 * tile + 2];
@@ -517,7 +549,7 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
       acc = fmaf(xv, to_float(wr[k]), acc);
       if (GATED) acc2 = fmaf(xv, to_float(wr[static_cast<int64_t>(N) * K + k]), acc2);
     }
-    out[out_row * out_stride + n] = from_float<TO>(GATED ? clamped_glu(acc, acc2, limit, alpha) : acc);
+    out[out_row * out_stride + n] = from_float<TO>(GATED ? clamped_glu(acc, acc2, limit, alpha, shift) : acc);
   }
 }
 
@@ -539,40 +571,48 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ ou
 
 template <typename T>
 __global__ __launch_bounds__(256) void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ gate_up,
-                                                          int64_t n, int I, float limit, float alpha) {
+                                                          int64_t n, int I, float limit, float alpha, float shift) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const int64_t t = idx / I, i = idx - t * I;
   const T* row = gate_up + t * 2 * I;
-  out[idx] = from_float<T>(clamped_glu(to_float(row[i]), to_float(row[I + i]), limit, alpha));
+  out[idx] = from_float<T>(clamped_glu(to_float(row[i]), to_float(row[I + i]), limit, alpha, shift));
 }
 
 }  // namespace
 
 extern "C" int kvc_moe_route(int32_t* choice, float* weight, const float* logits, int T, int E, int top,
-                             int groups, int keep, kvc_stream stream) {
+                             int groups, int keep, int score_fn, const float* correction, int group_best,
+                             float weight_scale, kvc_stream stream) {
   if (T < 0 || E <= 0 || top <= 0 || top > E || top > kWave || groups <= 0 || E % groups || keep <= 0 ||
       keep > groups)
     return kvc_fail("kvc_moe_route: bad sizes (at most 64 choices; the experts in equal groups)");
-  const size_t lds = sizeof(float) * 4 * (E + groups);
+  if ((score_fn != 0 && score_fn != 1) || (group_best != 1 && group_best != 2))
+    return kvc_fail("kvc_moe_route: scores by softmax (0) or sigmoid (1); a group is worth its best 1 or 2");
+  const RouteRule rule{top, groups, keep, score_fn, group_best, correction, weight_scale};
+  const size_t lds = sizeof(float) * 4 * (2 * E + groups);
   if (lds > 60000) return kvc_fail("kvc_moe_route: too many experts for a wave's scores in LDS");
   if (T == 0) return 0;
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), lds, S(stream), choice, weight, logits, T, E,
-                     top, groups, keep);
+                     rule);
   return kvc_check_launch("kvc_moe_route");
 }
 
 extern "C" int kvc_moe_router(int32_t* choice, float* weight, const void* x, int64_t x_stride, int x_dtype,
                               const float* router, int T, int H, int E, int top, int groups, int keep,
+                              int score_fn, const float* correction, int group_best, float weight_scale,
                               kvc_stream stream) {
   if (T < 0 || H <= 0 || E <= 0 || top <= 0 || top > E || top > kWave || groups <= 0 || E % groups || keep <= 0 ||
       keep > groups || x_stride < H)
     return kvc_fail("kvc_moe_router: bad sizes (at most 64 choices; the experts in equal groups)");
+  if ((score_fn != 0 && score_fn != 1) || (group_best != 1 && group_best != 2))
+    return kvc_fail("kvc_moe_router: scores by softmax (0) or sigmoid (1); a group is worth its best 1 or 2");
+  const RouteRule rule{top, groups, keep, score_fn, group_best, correction, weight_scale};
   if (T == 0) return 0;
   // four tokens a block where the blocks then still fill the chip several times over, else one
   const bool big = T >= 4 * 8 * kvc_device_compute_units();
   const int TOK = big ? 4 : 1;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(256) * 33 + static_cast<size_t>(TOK) * (E + groups));
+  const size_t lds = sizeof(float) * (static_cast<size_t>(256) * 33 + static_cast<size_t>(TOK) * (2 * E + groups));
   if (lds > 160 * 1024) return kvc_fail("kvc_moe_router: too many experts for a block's LDS");
   const dim3 grid((T + TOK - 1) / TOK);
   // 16-byte loads of the router's rows where the rows allow
@@ -585,7 +625,7 @@ extern "C" int kvc_moe_router(int32_t* choice, float* weight, const void* x, int
       if (attr != hipSuccess) return kvc_fail("kvc_moe_router: the kernel's LDS size was refused");            \
     }                                                                                                           \
     hipLaunchKernelGGL((moe_router_kernel<Tp, TOK_>), grid, dim3(256), lds, S(stream), choice, weight,          \
-                       static_cast<const Tp*>(x), x_stride, router, T, H, E, top, groups, keep, vectors);       \
+                       static_cast<const Tp*>(x), x_stride, router, T, H, E, rule, vectors);             \
   } while (0)
   if (x_dtype == 1 && big) KVC_ROUTER(bf16_t, 4);
   else if (x_dtype == 1) KVC_ROUTER(bf16_t, 1);
@@ -619,14 +659,15 @@ extern "C" int kvc_moe_align(int32_t* sorted, int32_t* tiles, int32_t* num_tiles
 extern "C" int kvc_moe_gemm(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride,
                             const void* w, int dtype, const int32_t* sorted, const int32_t* tiles,
                             const int32_t* num_tiles, int max_tiles, int tile_rows, int N, int K, int in_div,
-                            int out_sorted, int gated, float limit, float alpha, int packed, kvc_stream stream) {
+                            int out_sorted, int gated, float limit, float alpha, float up_shift, int packed,
+                            kvc_stream stream) {
   if (max_tiles < 0 || N <= 0 || K <= 0 || x_stride < K || out_stride < N)
     return kvc_fail("kvc_moe_gemm: bad sizes");
   if (tile_rows != kTileRows && tile_rows != kBigTileRows) return kvc_fail("kvc_moe_gemm: tiles of 16 or 64 rows");
   if (max_tiles == 0) return 0;
   dim3 grid(max_tiles, (N + 63) / 64);
   if (grid.y > 65535u) return kvc_fail("kvc_moe_gemm: too many columns");
-#define KVC_MOE_ARGS sorted, tiles, num_tiles, N, K, in_div, out_sorted, limit, alpha
+#define KVC_MOE_ARGS sorted, tiles, num_tiles, N, K, in_div, out_sorted, limit, alpha, up_shift
 #define KVC_MOE_LAUNCH(KERNEL, TI, TO)                                                                          \
   hipLaunchKernelGGL(KERNEL, grid, dim3(256), 0, S(stream), static_cast<TO*>(out), out_stride,                   \
                      static_cast<const TI*>(x), x_stride, static_cast<const TI*>(w), KVC_MOE_ARGS)
@@ -707,6 +748,6 @@ extern "C" int kvc_clamped_glu(void* out, const void* gate_up, int T, int I, flo
   const dim3 grid(static_cast<unsigned>((n + 255) / 256));
   KVC_DISPATCH_DTYPE(dtype, Tp,
                      hipLaunchKernelGGL((clamped_glu_kernel<Tp>), grid, dim3(256), 0, S(stream),
-                                        static_cast<Tp*>(out), static_cast<const Tp*>(gate_up), n, I, limit, alpha));
+                                        static_cast<Tp*>(out), static_cast<const Tp*>(gate_up), n, I, limit, alpha, 1.f));
   return kvc_check_launch("kvc_clamped_glu");
 }

@@ -253,6 +253,30 @@ __global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ out, con
   out[idx] = from_float<T>(to_float(x[t * x_stride + static_cast<int64_t>(h) * head_stride + skip + e]) * g);
 }
 
+// Two softmax maps a head over the same values: rows of attn are [heads][2][dv]; the second map is
+// taken off the first lambda times, the difference divided by its root mean square over the
+// head's dv values (eps inside the root, no gain) and multiplied by post.  A wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void diff_heads_norm_kernel(T* __restrict__ out, const T* __restrict__ attn,
+                                                              int64_t attn_stride, float lambda, float eps,
+                                                              float post, int64_t pairs, int heads, int dv) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t th = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (th >= pairs) return;  // the whole wave
+  const int64_t t = th / heads;
+  const int h = static_cast<int>(th - t * heads);
+  const T* a1 = attn + t * attn_stride + static_cast<int64_t>(2 * h) * dv;
+  const T* a2 = a1 + dv;
+  float ss = 0.f;
+  for (int e = lane; e < dv; e += kWave) {
+    const float o = to_float(a1[e]) - lambda * to_float(a2[e]);
+    ss += o * o;
+  }
+  const float inv = rsqrtf(wave_sum(ss) / static_cast<float>(dv) + eps) * post;
+  T* o_row = out + th * dv;
+  for (int e = lane; e < dv; e += kWave) o_row[e] = from_float<T>((to_float(a1[e]) - lambda * to_float(a2[e])) * inv);
+}
+
 }  // namespace
 
 extern "C" int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* delta, int delta_dtype,
@@ -297,10 +321,11 @@ extern "C" int kvc_wide_qk_norm(void* qkv, int64_t stride, const float* q_gain, 
 extern "C" int kvc_latent_rows(void* cq, int64_t cq_stride, void* key, void* value, int64_t kv_stride,
                                const void* down, int64_t down_stride, const float* q_gain, const float* kv_gain,
                                float eps, int T, int q_rank, int rank, int rot, int dtype, kvc_stream stream) {
-  if (T < 0 || q_rank <= 0 || rank <= 0 || rot < 0 || cq_stride < q_rank || kv_stride < rank + rot ||
+  if (T < 0 || q_rank < 0 || rank <= 0 || rot < 0 || cq_stride < q_rank || kv_stride < rank + rot ||
       down_stride < static_cast<int64_t>(q_rank) + rank + rot)
     return kvc_fail("kvc_latent_rows: rows too short for the sections");
-  if (cq == nullptr || key == nullptr || value == nullptr || down == nullptr || q_gain == nullptr || kv_gain == nullptr)
+  if (key == nullptr || value == nullptr || down == nullptr || kv_gain == nullptr ||
+      (q_rank > 0 && (cq == nullptr || q_gain == nullptr)))
     return kvc_fail("kvc_latent_rows: null operand");
   if (T == 0) return 0;
   KVC_DISPATCH_DTYPE(dtype, Tp,
@@ -325,4 +350,19 @@ extern "C" int kvc_head_gate(void* out, const void* x, int64_t x_stride, const v
                                         static_cast<const Tp*>(gate), gate_stride,
                                         total, heads, head_stride, skip, n));
   return kvc_check_launch("kvc_head_gate");
+}
+
+extern "C" int kvc_diff_heads_norm(void* out, const void* attn, int64_t attn_stride, float lambda, float eps, float post,
+                                   int T, int heads, int dv, int dtype, kvc_stream stream) {
+  if (T < 0 || heads <= 0 || dv <= 0 || attn_stride < static_cast<int64_t>(2) * heads * dv)
+    return kvc_fail("kvc_diff_heads_norm: bad sizes");
+  if (out == nullptr || attn == nullptr) return kvc_fail("kvc_diff_heads_norm: null operand");
+  const int64_t pairs = static_cast<int64_t>(T) * heads;
+  if (pairs == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((pairs + 3) / 4);
+  KVC_DISPATCH_DTYPE(dtype, Tp,
+                     hipLaunchKernelGGL(diff_heads_norm_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),
+                                        static_cast<Tp*>(out), static_cast<const Tp*>(attn), attn_stride, lambda, eps,
+                                        post, pairs, heads, dv));
+  return kvc_check_launch("kvc_diff_heads_norm");
 }

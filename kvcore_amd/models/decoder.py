@@ -102,6 +102,13 @@ class DecoderModel:
         for _, part in self._owned:
             part.setup(self.runtime)
 
+        # a block arrangement may keep several copies of every token's row in the stream
+        self.stream_copies = max((block.stream_copies for block in self.blocks), default=1)
+        if any(block.stream_copies != self.stream_copies for block in self.blocks):
+            raise ValueError("the blocks of a model keep the same number of copies of the stream")
+        if self.stream_copies > 1 and (self.stream_ops or any(type(pe).embed is not parts.PositionEncoding.embed
+                                                              for pe in self.positions)):
+            raise ValueError("stream ops and position encodings that rewrite the stream take a stream of one copy")
         self._plan_caches()
         self.params: dict[str, BoundParam] = {}
         self._allocate_params()
@@ -262,8 +269,14 @@ class DecoderModel:
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Normalised hidden rows ``[T, H]`` in the model dtype for the batch in ``ctx``."""
         H = self.spec.hidden_size
-        residual = ctx.buf("residual", H, torch.float32)
-        self.embed.forward(residual, ctx.token_ids[: ctx.num_tokens])
+        if self.stream_copies == 1:
+            residual = ctx.buf("residual", H, torch.float32)
+            self.embed.forward(residual, ctx.token_ids[: ctx.num_tokens])
+        else:  # every copy starts as the embedding's row
+            first = ctx.buf("embedded_rows", H, torch.float32)
+            self.embed.forward(first, ctx.token_ids[: ctx.num_tokens])
+            residual = ctx.buf(f"residual:{self.stream_copies}", self.stream_copies * H, torch.float32)
+            ops.spread_streams(residual, first, self.stream_copies)
         for pe in self.positions:
             pe.prepare(ctx)
             pe.embed(residual, ctx)
@@ -276,9 +289,7 @@ class DecoderModel:
             entry = self.schedule[i]
             if entry.before is not None:
                 if delta is not None:  # what the layer before left pending joins the stream first
-                    if isinstance(delta, (ops.ScaledRows, ops.NormedRows)):
-                        raise RuntimeError("a stream op follows a block that folded the next norm")
-                    ops.residual_add(residual, delta)
+                    self.blocks[self.calls[i - 1].layer_index].settle(delta, residual, ctx)
                     delta = None
                 self.stream_ops[entry.before].forward(residual, embedded, ctx, entry.before_arg)
             # a block may leave its last sum and the next block's first norm to the products
@@ -288,7 +299,10 @@ class DecoderModel:
                 nxt = self.blocks[self.calls[i + 1].layer_index]
             delta = self.blocks[call.layer_index].forward(delta, residual, ctx, call, next_block=nxt)
         hidden = ctx.buf("final_hidden", H)
-        self.final_norm.forward_fused(hidden, residual, delta)
+        if self.calls:
+            self.blocks[self.calls[-1].layer_index].finish(delta, residual, ctx, self.final_norm, hidden)
+        else:
+            self.final_norm.forward_fused(hidden, residual, delta)
         return hidden
 
     def compute_logits(self, ctx: StepContext, hidden: torch.Tensor, rows: torch.Tensor,

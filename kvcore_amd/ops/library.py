@@ -43,6 +43,10 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_residual_add2": [P, P, I, P, I, I, I, P],
         "kvc_silu_mul": [P, P, I, I, I, P],
         "kvc_gate_mul": [P, P, I, I, I, I, P],
+        "kvc_activation": [P, P, L, I, I, P],
+        "kvc_hyper_step": [P, I, P, P, I, P, P, F, P, P, F, I, I, I, P],
+        "kvc_spread_streams": [P, P, I, I, I, P],
+        "kvc_diff_heads_norm": [P, P, L, F, F, F, I, I, I, I, P],
         "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, I, P],
         "kvc_wide_qk_norm": [P, L, P, P, F, I, I, I, I, I, P],
         "kvc_head_gate": [P, P, L, P, L, I, I, I, I, I, I, P],
@@ -60,12 +64,12 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_decay_and_write_gates": [P, P, P, L, P, L, P, P, I, I, P],
         "kvc_unit_heads": [P, L, I, I, I, F, F, I, F, P],
         "kvc_head_rmsnorm_gate": [P, I, P, P, L, I, P, F, I, I, I, P],
-        "kvc_moe_route": [P, P, P, I, I, I, I, I, P],
-        "kvc_moe_router": [P, P, P, L, I, P, I, I, I, I, I, I, P],
+        "kvc_moe_route": [P, P, P, I, I, I, I, I, I, P, I, F, P],
+        "kvc_moe_router": [P, P, P, L, I, P, I, I, I, I, I, I, I, P, I, F, P],
         "kvc_moe_max_tiles": [I, I, I],
         "kvc_moe_tile_rows": [I, I],
         "kvc_moe_align": [P, P, P, P, I, I, I, I, P],
-        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
+        "kvc_moe_gemm": [P, L, I, P, L, P, I, P, P, P, I, I, I, I, I, I, I, F, F, F, I, P],
         "kvc_moe_combine": [P, P, P, I, P, I, P, I, I, I, P],
         "kvc_clamped_glu": [P, P, I, I, F, F, I, P],
         "kvc_qk_norm_rope_kv_write": [P, L, P, P, I, P, P, F, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
@@ -301,6 +305,98 @@ def silu_mul(out: torch.Tensor, gate_up: torch.Tensor, act: str = "silu") -> Non
         raise KernelError("silu_mul: shapes or dtypes do not match")
     _check(load().kvc_gate_mul(_dev(out, "out"), _dev(gate_up, "gate_up"), T, I2 // 2, _gate_act(act),
                                _code(out, "out"), _stream()), "kvc_gate_mul")
+
+
+ACTIVATIONS = {"relu_squared": 0}  # activations of a feed-forward without a gate
+
+
+def activation(out: torch.Tensor, x: torch.Tensor, act: str) -> None:
+    """``out = act(x)`` elementwise (in place is fine); ``act``: ``relu_squared``."""
+    if act not in ACTIVATIONS:
+        raise KernelError(f"unknown activation {act!r} (known: {sorted(ACTIVATIONS)})")
+    if out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous() or not x.is_contiguous():
+        raise KernelError("activation: shapes or dtypes do not match")
+    _check(load().kvc_activation(_dev(out, "out"), _dev(x, "x"), x.numel(), ACTIVATIONS[act], _code(x, "x"),
+                                 _stream()), "kvc_activation")
+
+
+HYPER_MAX_COPIES = 8
+
+
+def hyper_step(out: torch.Tensor | None, streams: torch.Tensor, copies: int, y: torch.Tensor | None = None, *,
+               mix: torch.Tensor | None = None, out_w: torch.Tensor | None = None, mult: float = 1.0,
+               in_w: torch.Tensor | None = None, gain: torch.Tensor | None = None, eps: float = 0.0) -> None:
+    """One step of a residual stream kept as ``copies`` rows a token (``streams [T, copies * H]``
+    float32).  With ``y [T, H]``: every copy at once from the old ones, ``x_t <- sum_s mix[s, t] x_s
+    + mult * out_w[t] * y`` (``mix`` None: the identity, ``out_w`` None: ones).  Then, with ``out
+    [T, H]``: ``u = sum_t in_w[t] x_t`` (``in_w`` None: ones) and ``out = gain * u / sqrt(mean(u^2)
+    + eps)``.  One copy and no coefficients: ``x += mult * y`` and the norm."""
+    T = streams.shape[0]
+    if copies < 1 or streams.shape[1] % copies or streams.dtype != torch.float32 or not streams.is_contiguous():
+        raise KernelError("hyper_step: the stream is contiguous float32 [T, copies * H]")
+    H = streams.shape[1] // copies
+    for t, name in ((y, "y"), (out, "out")):
+        if t is not None and (t.shape != (T, H) or not t.is_contiguous()):
+            raise KernelError(f"hyper_step: {name} must be contiguous [T, H]")
+    for t, n, name in ((mix, copies * copies, "mix"), (out_w, copies, "out_w"), (in_w, copies, "in_w"), (gain, H, "gain")):
+        if t is not None and (t.numel() != n or t.dtype != torch.float32 or not t.is_contiguous()):
+            raise KernelError(f"hyper_step: {name} must be float32 with {n} values")
+    if out is not None and gain is None:
+        raise KernelError("hyper_step: the norm needs its gain")
+    _check(load().kvc_hyper_step(
+        None if out is None else _dev(out, "out"), 0 if out is None else _code(out, "out"), _dev(streams, "streams"),
+        None if y is None else _dev(y, "y"), 0 if y is None else _code(y, "y"),
+        None if mix is None else _dev(mix, "mix"), None if out_w is None else _dev(out_w, "out_w"), float(mult),
+        None if in_w is None else _dev(in_w, "in_w"), None if gain is None else _dev(gain, "gain"), float(eps),
+        T, H, copies, _stream()), "kvc_hyper_step")
+
+
+@dataclass
+class StreamWrite:
+    """A sublayer's result ``y [T, H]`` that has still to join a stream of ``copies`` rows a token:
+    ``x_t <- sum_s mix[s, t] x_s + mult * out_w[t] * y`` (see :func:`hyper_step`)."""
+
+    y: torch.Tensor
+    copies: int
+    mix: torch.Tensor | None
+    out_w: torch.Tensor | None
+    mult: float
+
+
+def stream_write_read(out: torch.Tensor | None, streams: torch.Tensor, copies: int, pending: StreamWrite | None, *,
+                      in_w: torch.Tensor | None = None, gain: torch.Tensor | None = None, eps: float = 0.0) -> None:
+    """The pending write (may be None) and the next read with its norm (``out`` None: no read) in
+    one pass over the copies."""
+    if pending is None:
+        if out is not None:
+            hyper_step(out, streams, copies, in_w=in_w, gain=gain, eps=eps)
+        return
+    if pending.copies != copies:
+        raise KernelError("stream_write_read: the pending result was made for another number of copies")
+    hyper_step(out, streams, copies, pending.y, mix=pending.mix, out_w=pending.out_w, mult=pending.mult,
+               in_w=in_w, gain=gain, eps=eps)
+
+
+def spread_streams(streams: torch.Tensor, rows: torch.Tensor, copies: int) -> None:
+    """``streams[t, c, :] = rows[t, :]`` for every copy ``c``: all copies start as the same row."""
+    T, H = rows.shape
+    if streams.shape != (T, copies * H) or streams.dtype != torch.float32 or rows.dtype != torch.float32 \
+            or not streams.is_contiguous() or not rows.is_contiguous():
+        raise KernelError("spread_streams: float32 [T, copies * H] from float32 [T, H]")
+    _check(load().kvc_spread_streams(_dev(streams, "streams"), _dev(rows, "rows"), T, H, copies, _stream()),
+           "kvc_spread_streams")
+
+
+def diff_heads_norm(out: torch.Tensor, attn: torch.Tensor, *, heads: int, dv: int, lam: float, eps: float,
+                    post: float) -> None:
+    """Rows of ``attn`` hold ``heads`` pairs of results ``[a1 | a2]`` of ``dv`` values each; ``out[t,
+    h] = (a1 - lam * a2) / sqrt(mean((a1 - lam * a2)^2) + eps) * post`` over the head's ``dv`` values."""
+    T = out.shape[0]
+    if out.shape != (T, heads * dv) or not out.is_contiguous() or attn.shape[0] < T or attn.stride(1) != 1 \
+            or attn.shape[1] < 2 * heads * dv or attn.dtype != out.dtype:
+        raise KernelError("diff_heads_norm: shapes do not match")
+    _check(load().kvc_diff_heads_norm(_dev(out, "out"), attn.data_ptr(), attn.stride(0), float(lam), float(eps),
+                                      float(post), T, heads, dv, _code(out, "out"), _stream()), "kvc_diff_heads_norm")
 
 
 def gather_rows(out: torch.Tensor, src: torch.Tensor, rows: torch.Tensor) -> None:
@@ -1510,21 +1606,26 @@ def wide_qk_norm(qkv: torch.Tensor, q_gain: torch.Tensor, k_gain: torch.Tensor, 
                                    int(bool(copy_k)), _code(qkv, "qkv"), _stream()), "kvc_wide_qk_norm")
 
 
-def latent_rows(cq: torch.Tensor, key: torch.Tensor, value: torch.Tensor, down: torch.Tensor, q_gain: torch.Tensor,
-                kv_gain: torch.Tensor, eps: float, rot: int) -> None:
+def latent_rows(cq: torch.Tensor | None, key: torch.Tensor, value: torch.Tensor, down: torch.Tensor,
+                q_gain: torch.Tensor | None, kv_gain: torch.Tensor, eps: float, rot: int) -> None:
     """From rows ``down = [query latent | key/value latent | rot rotated key elements | ...]``: the
     query latent normed with ``q_gain`` into ``cq``; ``[rotated elements as they are | key/value
     latent normed with kv_gain]`` into ``key`` and into ``value`` (column views of one buffer with
     equal row strides are fine).  All of one dtype; the norms are float32."""
     T = down.shape[0]
-    q_rank, rank = q_gain.numel(), kv_gain.numel()
+    q_rank, rank = (0 if q_gain is None else q_gain.numel()), kv_gain.numel()
+    if (cq is None) != (q_gain is None):
+        raise KernelError("latent_rows: a query latent has rows and a gain, or neither")
     for t, cols in ((cq, q_rank), (key, rank + rot), (value, rank + rot)):
+        if t is None:
+            continue
         if t.dim() != 2 or t.shape != (T, cols) or t.stride(1) != 1 or t.dtype != down.dtype:
             raise KernelError("latent_rows: results do not fit")
     if down.stride(1) != 1 or down.shape[1] < q_rank + rank + rot or key.stride(0) != value.stride(0):
         raise KernelError("latent_rows: rows too short, or keys and values with different strides")
-    _check(load().kvc_latent_rows(cq.data_ptr(), cq.stride(0), key.data_ptr(), value.data_ptr(), key.stride(0),
-                                  down.data_ptr(), down.stride(0), _dev(q_gain, "q_gain", torch.float32),
+    _check(load().kvc_latent_rows(None if cq is None else cq.data_ptr(), 0 if cq is None else cq.stride(0),
+                                  key.data_ptr(), value.data_ptr(), key.stride(0), down.data_ptr(), down.stride(0),
+                                  None if q_gain is None else _dev(q_gain, "q_gain", torch.float32),
                                   _dev(kv_gain, "kv_gain", torch.float32), float(eps), T, q_rank, rank, int(rot),
                                   _code(down, "down"), _stream()), "kvc_latent_rows")
 
@@ -1545,20 +1646,41 @@ def head_gate(out: torch.Tensor, x: torch.Tensor, gate: torch.Tensor, *, heads: 
                                 _code(out, "out"), _stream()), "kvc_head_gate")
 
 
+ROUTE_SCORES = {"softmax": 0, "sigmoid": 1}  # how a router's logits become scores
+
+
+def _route_rule(E: int, score: str, correction: torch.Tensor | None, group_best: int,
+                weight_scale: float) -> tuple[int, int | None, int, float]:
+    if score not in ROUTE_SCORES:
+        raise KernelError(f"unknown router score {score!r} (known: {sorted(ROUTE_SCORES)})")
+    if correction is not None and (correction.shape != (E,) or correction.dtype != torch.float32):
+        raise KernelError("moe routing: the correction is float32 [experts]")
+    if group_best not in (1, 2):
+        raise KernelError("moe routing: a group is worth its best choice score or the sum of its best two")
+    return (ROUTE_SCORES[score], None if correction is None else _dev(correction, "correction"), int(group_best),
+            float(weight_scale))
+
+
 def moe_route(choice: torch.Tensor, weight: torch.Tensor, logits: torch.Tensor, *, top: int, groups: int = 1,
-              keep: int = 1) -> None:
+              keep: int = 1, score: str = "softmax", correction: torch.Tensor | None = None, group_best: int = 1,
+              weight_scale: float = 1.0) -> None:
     """The router's choice from float32 ``logits [T, E]``: ``choice`` (int32) and ``weight``
-    (float32), both ``[T, top]`` (see the C header for the rule)."""
+    (float32), both ``[T, top]``.  ``score``: ``softmax`` over the experts or a ``sigmoid`` of each
+    logit; ``correction`` (float32 ``[E]``) joins the scores for the choice alone; a group is worth
+    its ``group_best`` (1 or 2) best choice scores; the weights (the chosen experts' plain scores
+    over their sum) are multiplied by ``weight_scale``."""
     T, E = logits.shape
     if choice.shape != (T, top) or weight.shape != (T, top):
         raise KernelError("moe_route: shapes do not match")
     _check(load().kvc_moe_route(_dev(choice, "choice", torch.int32), _dev(weight, "weight", torch.float32),
-                                _dev(logits, "logits", torch.float32), T, E, top, groups, keep, _stream()),
+                                _dev(logits, "logits", torch.float32), T, E, top, groups, keep,
+                                *_route_rule(E, score, correction, group_best, weight_scale), _stream()),
            "kvc_moe_route")
 
 
 def moe_router(choice: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, router: torch.Tensor, *, top: int,
-               groups: int = 1, keep: int = 1) -> None:
+               groups: int = 1, keep: int = 1, score: str = "softmax", correction: torch.Tensor | None = None,
+               group_best: int = 1, weight_scale: float = 1.0) -> None:
     """``moe_route`` of the logits ``x @ router.T`` (float32 sums in one fixed order; ``x [T, H]`` of
     either dtype, ``router [E, H]`` float32) without storing the logits."""
     T, H = x.shape
@@ -1567,7 +1689,9 @@ def moe_router(choice: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rout
         raise KernelError("moe_router: shapes do not match")
     _check(load().kvc_moe_router(_dev(choice, "choice", torch.int32), _dev(weight, "weight", torch.float32),
                                  x.data_ptr(), x.stride(0), _code(x, "x"), _dev(router, "router", torch.float32),
-                                 T, H, E, top, groups, keep, _stream()), "kvc_moe_router")
+                                 T, H, E, top, groups, keep,
+                                 *_route_rule(E, score, correction, group_best, weight_scale), _stream()),
+           "kvc_moe_router")
 
 
 def moe_tile_rows(pairs: int, experts: int, x: torch.Tensor | None = None, k_sizes: tuple[int, ...] = ()) -> int:
@@ -1597,9 +1721,10 @@ def moe_align(sorted_pairs: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.
 
 def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tiles: torch.Tensor,
              num_tiles: torch.Tensor, *, pairs: int, experts: int, in_div: int, out_sorted: bool, gated: bool,
-             limit: float = 0.0, alpha: float = 0.0, tile_rows: int = 16) -> None:
+             limit: float = 0.0, alpha: float = 0.0, up_shift: float = 1.0, tile_rows: int = 16) -> None:
     """Every expert's product over its own rows.  ``w`` is ``[experts * N, K]`` (``experts * 2N``
-    rows when ``gated``: each expert's gate rows, then its up rows); ``out [pairs, N]``."""
+    rows when ``gated``: each expert's gate rows, then its up rows); ``out [pairs, N]``.  The gated
+    form stores ``min(g, limit) * sigmoid(alpha * g) * (clamp(u, -limit, limit) + up_shift)``."""
     N = out.shape[1]
     K = x.shape[1]
     rows = experts * N * (2 if gated else 1)
@@ -1612,7 +1737,7 @@ def moe_gemm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, sorted_pairs: 
                                w_ptr, _code(x, "x"), _dev(sorted_pairs, "sorted", torch.int32),
                                _dev(tiles, "tiles", torch.int32), _dev(num_tiles, "num_tiles", torch.int32),
                                max_tiles, tile_rows, N, K, int(in_div), int(bool(out_sorted)), int(bool(gated)),
-                               float(limit), float(alpha), packed, _stream()), "kvc_moe_gemm")
+                               float(limit), float(alpha), float(up_shift), packed, _stream()), "kvc_moe_gemm")
 
 
 def moe_combine(out: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, add0: torch.Tensor | None = None,

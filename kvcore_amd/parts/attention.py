@@ -436,4 +436,83 @@ def _sized(name: str, cols: int, plain: bool) -> str:
     return name if plain else f"{name}:{cols}"
 
 
+class DifferentialAttention(PagedAttention):
+    """Grouped-query attention with two softmax maps a head over the same values: ``o = a1 - lambda
+    * a2``, then each head's ``o`` over its root mean square (``eps`` inside the root, no gain) times
+    ``1 - diff``, then the output product.  ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff`` is one
+    number for the layer, from four learned vectors of ``head_dim`` values.
+
+    The checkpoint's q and k hold, head by head, the two maps' parts ``[map 1 | map 2]``.  A kv
+    head's two key parts are kept as ONE cached key of ``2 * head_dim`` values, and every query head
+    becomes two heads of that size, ``[q1 | 0]`` and ``[0 | q2]``: their scores against the joint key
+    are the two maps' scores, so the layer is the paged attention of this file with ``2 * heads``
+    query heads over ``kv_heads`` key/value heads (a token's keys and values are stored and read
+    once for both maps), followed by one small kernel that joins the maps.  The zeros are rows of
+    the fused projection matrix made when the weights arrive.  ``tensor_names`` renames checkpoint
+    tensors (keys ``q``, ``k``, ``v``, ``o``, ``lq1``, ``lk1``, ``lq2``, ``lk2``)."""
+
+    any_head_size = True
+    takes_sink = False  # the maps are joined between the attention and the output product's input
+
+    def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
+                 scale: float, diff: float, eps: float, window: int = 0, page_size: int | None = None,
+                 tensor_names: dict[str, str] | None = None, float32_result: bool = False,
+                 position: PositionEncoding | None = None) -> None:
+        if position is not None:
+            raise ValueError("differential attention rotates nothing: the zero halves of its query heads "
+                             "must stay zero")
+        super().__init__(hidden_size=hidden_size, num_heads=2 * num_heads, num_kv_heads=num_kv_heads,
+                         head_dim=2 * head_dim, v_head_dim=v_head_dim, scale=scale, window=window,
+                         page_size=page_size, float32_result=float32_result, sized_buffers=True)
+        self.heads, self.map_dim, self.diff, self.eps = num_heads, head_dim, float(diff), float(eps)
+        self.map_names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                          "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2", "lk2": "lambda_k2",
+                          **(tensor_names or {})}
+        self.lam: float | None = None
+
+    def param_specs(self) -> list[ParamSpec]:
+        n, H, d = self.map_names, self.hidden_size, self.map_dim
+
+        def one(name: str, key: str, shape: tuple[int, ...], **kw) -> ParamSpec:
+            return ParamSpec(name, shape, sources=(ParamSource(n[key], 0, shape[0]),), **kw)
+
+        return [
+            one("q.weight", "q", (self.heads * 2 * d, H)),
+            one("k.weight", "k", (self.kv_size, H)),
+            one("v.weight", "v", (self.v_size, H)),
+            one("o_proj.weight", "o", (H, self.heads * self.v_head_dim)),
+            *[one(key, key, (d,), kind="vector") for key in ("lq1", "lk1", "lq2", "lk2")],
+        ]
+
+    def weights_loaded(self) -> None:
+        """The fused projection ``[padded q heads | k | v]`` and the layer's ``lambda``."""
+        p, d = self.params, self.map_dim
+        q = p["q.weight"].view(self.heads, 2, d, self.hidden_size)
+        padded = torch.zeros(self.heads, 2, 2, d, self.hidden_size, dtype=q.dtype, device=q.device)
+        padded[:, 0, 0] = q[:, 0]  # head 2h: [q1 | 0]
+        padded[:, 1, 1] = q[:, 1]  # head 2h + 1: [0 | q2]
+        fused = torch.cat([padded.view(self.q_size, self.hidden_size), p["k.weight"], p["v.weight"]], dim=0)
+        old = p.get("qkv_proj.weight")
+        if old is None:
+            p["qkv_proj.weight"] = fused.contiguous()
+        else:  # weights loaded again: the same storage, so nothing that holds it goes stale
+            old.copy_(fused)
+            if hasattr(old, "kvc_packed"):
+                del old.kvc_packed
+        f = torch.float32
+        lam = torch.exp((p["lq1"].to(f) * p["lk1"].to(f)).sum()) - torch.exp((p["lq2"].to(f) * p["lk2"].to(f)).sum())
+        self.lam = float(lam.item()) + self.diff
+
+    def forward(self, x, ctx, call, sink=None):
+        if "qkv_proj.weight" not in self.params or self.lam is None:
+            self.weights_loaded()
+        maps = self._attention(self._project(x, ctx), ctx, call)  # [T, heads x (a1 | a2)]
+        width = self.heads * self.v_head_dim
+        joined = ctx.buf(f"attn_joined:{width}", width)
+        ops.diff_heads_norm(joined, maps, heads=self.heads, dv=self.v_head_dim, lam=self.lam, eps=self.eps,
+                            post=1.0 - self.diff)
+        return self._output(joined, ctx, sink)
+
+
 register_mixer("paged_attention", PagedAttention)
+register_mixer("differential_attention", DifferentialAttention)

@@ -332,6 +332,26 @@ class Block(Part):
         slices = ctx.buffers.get("block_slices", ops.mid_slices_bound(H) * ops.MID_ROWS, H, torch.float32)
         return ops.ResidualSink(residual, gain[0], gain[1], rows, None, slices)
 
+    # how many copies of every token's row the residual stream holds for this arrangement (the
+    # model allocates ``[T, stream_copies * hidden]``; all blocks of a model agree)
+    stream_copies = 1
+
+    def settle(self, delta, residual: torch.Tensor, ctx: "StepContext") -> None:
+        """Add what a block of this kind left pending into the stream (before something other
+        than the next block reads it)."""
+        from kvcore_amd.ops import library as ops
+
+        if delta is not None:
+            if isinstance(delta, (ops.ScaledRows, ops.NormedRows)):
+                raise RuntimeError("a block that folded the next norm has nothing left to settle")
+            ops.residual_add(residual, delta)
+
+    def finish(self, delta, residual: torch.Tensor, ctx: "StepContext", final_norm: "Norm",
+               hidden: torch.Tensor) -> None:
+        """After the last block: the pending ``delta`` joins the stream and the model's final norm
+        writes ``hidden`` (model dtype)."""
+        final_norm.forward_fused(hidden, residual, delta)
+
     def input_gain(self, scaled: bool = True) -> "tuple[torch.Tensor, float] | None":
         """``(gain, eps)`` of the block's first norm (see :meth:`Norm.as_gain`) if the block
         before may do that norm's work, else None: with ``scaled`` it hands over

@@ -12,7 +12,7 @@ import torch
 
 from kvcore_amd.ops import library as ops
 
-from .base import Block, FeedForward, Mixer, Norm, Part, register_block
+from .base import Block, FeedForward, Mixer, Norm, ParamSource, ParamSpec, Part, register_block
 
 
 class PreNormBlock(Block):
@@ -220,6 +220,102 @@ class SandwichNormBlock(Block):
         return None if rows is None else ops.NormedRows(rows)
 
 
+class StreamLink(Part):
+    """How one sublayer hangs on a residual stream of several copies: ``in [copies]`` weighs the
+    copies into the sublayer's input, ``mix [copies, copies]`` (indexed [from, to]) carries the old
+    copies into the new ones, ``out [copies]`` weighs the sublayer's result into each.  All float32."""
+
+    def __init__(self, copies: int, names: tuple[str, str, str] = ("in", "mix", "out")) -> None:
+        self.copies, self.names = copies, names
+
+    def param_specs(self) -> list[ParamSpec]:
+        c, (n_in, n_mix, n_out) = self.copies, self.names
+        return [ParamSpec("in", (c,), kind="vector", init="gain", sources=(ParamSource(n_in, 0, c),)),
+                ParamSpec("mix", (c, c), kind="vector", init="mixing", sources=(ParamSource(n_mix, 0, c),)),
+                ParamSpec("out", (c,), kind="vector", init="gain", sources=(ParamSource(n_out, 0, c),))]
+
+
+class HyperConnectionBlock(Block):
+    """A pre-norm layer on a residual stream kept as ``copies`` rows a token, ``x_1 .. x_c``.  For
+    each sublayer f (mixer, then feed-forward) with its link (in, mix, out) and its norm:
+
+        u = sum_s in[s] x_s;   y = f(norm(u));   x_t <- sum_s mix[s, t] x_s + mult * out[t] * y
+
+    for all t at once from the old copies.  ``learned`` False: no link tensors, in = out = 1 and mix
+    the identity, which with one copy is the plain ``x <- x + mult * f(norm(x))``.  The write of one
+    sublayer and the read and norm of the next are one kernel (``ops.hyper_step``), across blocks
+    too: a block returns its last sublayer's result as a pending ``ops.StreamWrite``.  After the
+    last block the copies are added up and normed by the model's final norm.  The norms must be RMS
+    norms with a gain (``Norm.as_gain``).  With a feed-forward of kind ``none`` the layer is its
+    first half."""
+
+    def __init__(self, *, mixer: Mixer, ffn: FeedForward, norms: dict[str, Norm], copies: int = 1,
+                 learned: bool = True, mult: float = 1.0, mixer_name: str = "mixer", ffn_name: str = "mlp",
+                 mixer_norm: str = "norm1", ffn_norm: str = "norm2", mixer_link: str = "hc1",
+                 ffn_link: str = "hc2") -> None:
+        super().__init__(mixer=mixer, ffn=ffn, norms=norms)
+        if not 1 <= copies <= ops.HYPER_MAX_COPIES:
+            raise ValueError(f"a stream of {copies} copies (1 to {ops.HYPER_MAX_COPIES})")
+        self.stream_copies, self.learned, self.mult = int(copies), bool(learned), float(mult)
+        self.mixer_only = bool(getattr(ffn, "absent", False))
+        self.mixer_name, self.ffn_name = mixer_name, ffn_name
+        self.norm_names = (mixer_norm,) if self.mixer_only else (mixer_norm, ffn_norm)
+        missing = [n for n in self.norm_names if n not in norms]
+        if missing:
+            raise ValueError(f"this block needs the norms {self.norm_names}; given {list(norms)}")
+        self.link_names = (mixer_link, ffn_link)
+        self.links = [StreamLink(self.stream_copies) for _ in self.norm_names] if self.learned else []
+
+    def children(self) -> dict[str, Part]:
+        out: dict[str, Part] = {self.norm_names[0]: self.norms[self.norm_names[0]], self.mixer_name: self.mixer}
+        if not self.mixer_only:
+            out[self.norm_names[1]] = self.norms[self.norm_names[1]]
+            out[self.ffn_name] = self.ffn
+        for name, link in zip(self.link_names, self.links):
+            out[name] = link
+        return out
+
+    def _gain(self, i: int):
+        gain = self.norms[self.norm_names[i]].as_gain()
+        if gain is None:
+            raise RuntimeError(f"norm {self.norm_names[i]!r} is not an RMS norm with a gain")
+        return gain
+
+    def _written(self, y, i: int) -> "ops.StreamWrite":
+        """Sublayer i's result on its way into the copies."""
+        link = self.links[i].params if self.learned else {}
+        return ops.StreamWrite(y, self.stream_copies, link.get("mix"), link.get("out"), self.mult)
+
+    def _read(self, name: str, residual, ctx, pending, i: int):
+        """What is pending joins the copies; sublayer i's input, normed, into the step buffer ``name``."""
+        rows = ctx.buf(name, residual.shape[1] // self.stream_copies)
+        gain, eps = self._gain(i)
+        in_w = self.links[i].params["in"] if self.learned else None
+        ops.stream_write_read(rows, residual, self.stream_copies, pending, in_w=in_w, gain=gain, eps=eps)
+        return rows
+
+    def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
+        if delta is not None and not isinstance(delta, ops.StreamWrite):
+            raise RuntimeError("this block follows blocks of its own kind")
+        x = self._read("block_x", residual, ctx, delta, 0)
+        a = self.mixer.forward(x, ctx, call)
+        if self.mixer_only:
+            return self._written(a, 0)
+        x2 = self._read("block_x2", residual, ctx, self._written(a, 0), 1)
+        return self._written(self.ffn.forward(x2, ctx, call), 1)
+
+    def settle(self, delta, residual: torch.Tensor, ctx) -> None:
+        if delta is not None:
+            ops.stream_write_read(None, residual, self.stream_copies, delta)
+
+    def finish(self, delta, residual: torch.Tensor, ctx, final_norm: Norm, hidden: torch.Tensor) -> None:
+        gain = final_norm.as_gain()
+        if gain is None:
+            raise RuntimeError("the final norm of a stream of several copies is an RMS norm with a gain")
+        ops.stream_write_read(hidden, residual, self.stream_copies, delta, in_w=None, gain=gain[0], eps=gain[1])
+
+
 register_block("prenorm", PreNormBlock)
+register_block("hyper_connections", HyperConnectionBlock)
 register_block("sandwich_norm", SandwichNormBlock)
 register_block("parallel_residual", ParallelResidualBlock)

@@ -89,6 +89,54 @@ class SwiGLU(FeedForward):
         return out
 
 
+class DenseMLP(FeedForward):
+    """A feed-forward without a gate: ``down(act(up(x) + b_up)) + b_down``; ``activation`` is one of
+    ``ops.ACTIVATIONS`` (``relu_squared``: the square of relu), computed in float32 from the rows
+    as stored.  ``up_name``/``down_name`` are the checkpoint's names of the two matrices relative to
+    the part's prefix, ``suffix`` what follows each, ``bias_suffix`` what follows a bias."""
+
+    @property
+    def takes_scaled_rows(self) -> bool:  # x only goes into the up product
+        return self.hidden_size % 8 == 0
+
+    def __init__(self, *, hidden_size: int, intermediate_size: int, activation: str = "relu_squared",
+                 bias: bool = False, up_name: str = "up_proj", down_name: str = "down_proj",
+                 suffix: str = ".weight", bias_suffix: str = ".bias", float32_result: bool = False) -> None:
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not supported (supported: {sorted(ops.ACTIVATIONS)})")
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.activation, self.bias, self.float32_result = activation, bool(bias), float32_result
+        self.names, self.suffix, self.bias_suffix = (up_name, down_name), suffix, bias_suffix
+
+    def param_specs(self) -> list[ParamSpec]:
+        I, H = self.intermediate_size, self.hidden_size
+        up, down = self.names
+        specs = [ParamSpec("up_proj.weight", (I, H), sources=(ParamSource(up + self.suffix, 0, I),)),
+                 ParamSpec("down_proj.weight", (H, I), sources=(ParamSource(down + self.suffix, 0, H),))]
+        if self.bias:
+            # in the model's dtype, as the products' kernels take them
+            specs.append(ParamSpec("up_proj.bias", (I,), init="normal",
+                                   sources=(ParamSource(up + self.bias_suffix, 0, I),)))
+            specs.append(ParamSpec("down_proj.bias", (H,), init="normal",
+                                   sources=(ParamSource(down + self.bias_suffix, 0, H),)))
+        return specs
+
+    def product_weights(self) -> tuple[str, ...]:
+        return ("up_proj.weight", "down_proj.weight")
+
+    def forward(self, x, ctx, call, sink=None):
+        p, I = self.params, self.intermediate_size
+        act = ctx.buf(f"mlp_act:{I}", I)
+        ops.linear(act, x, p["up_proj.weight"], p.get("up_proj.bias"))
+        ops.activation(act, act, self.activation)
+        if self.float32_result:
+            out = ctx.buf("ffn_out_f32", self.hidden_size, torch.float32)
+        else:
+            out = ctx.buf("ffn_out", self.hidden_size)
+        ops.linear(out, act, p["down_proj.weight"], p.get("down_proj.bias"))
+        return out
+
+
 class NoFeedForward(FeedForward):
     """A layer that has a mixer only: the block skips the second norm and the second sum."""
 
@@ -99,4 +147,5 @@ class NoFeedForward(FeedForward):
 
 
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("mlp", DenseMLP)
 register_feed_forward("none", NoFeedForward)

@@ -77,5 +77,10 @@ def _register_builtin() -> None:
 
     register_architecture("Tazunex", TazunexConfig.from_dict, tazunex_spec)
 
+    from kvcore_amd.config.darovik_config import DarovikConfig
+    from kvcore_amd.models.darovik import darovik_spec
+
+    register_architecture("Darovik", DarovikConfig.from_dict, darovik_spec)
+
 
 _register_builtin()

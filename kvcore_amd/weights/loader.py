@@ -91,7 +91,7 @@ def load_weights(model: DecoderModel, model_dir: str | Path, *, strict: bool = T
 
 
 # ------------------------------------------------------------------- random weights
-_INIT_RULES = {"normal": (0.0, 0.02), "gain": (1.0, 0.1)}  # (mean, standard deviation)
+_INIT_RULES = {"normal": (0.0, 0.02), "gain": (1.0, 0.1), "mixing_noise": (0.0, 0.1)}  # (mean, standard deviation)
 
 
 def _tensor_seed(seed: int, name: str) -> tuple[int, int]:
@@ -106,7 +106,7 @@ def random_tensor(seed: int, name: str, shape: tuple[int, ...], init: str,
     index) only, so they depend neither on the order in which tensors are made, nor on how
     they are stacked, nor on the device that draws them (the GPU kernel and its host twin,
     ``weights/random_normal.py``, give the same bits).  ``normal``: N(0, 0.02); ``gain``:
-    1 + N(0, 0.1); ``zeros``."""
+    1 + N(0, 0.1); ``mixing``: a square matrix, the identity + N(0, 0.1); ``zeros``."""
     out = torch.empty(shape, dtype=torch.float32, device=device)
     fill_random(out, seed, name, init)
     return out
@@ -119,6 +119,12 @@ def fill_random(out: torch.Tensor, seed: int, name: str, init: str) -> None:
         raise ValueError("fill_random needs a contiguous tensor")
     if init == "zeros":
         out.zero_()
+        return
+    if init == "mixing":  # a square matrix near the identity
+        if out.dim() != 2 or out.shape[0] != out.shape[1]:
+            raise ValueError("the 'mixing' rule fills a square matrix")
+        fill_random(out, seed, name, "mixing_noise")
+        out.add_(torch.eye(out.shape[0], dtype=out.dtype, device=out.device))
         return
     mean, std = _INIT_RULES[init]
     lo, hi = _tensor_seed(seed, name)
