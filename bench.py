@@ -20,7 +20,8 @@ Other workloads print a line of their own: ``--only-prefill``, ``--mixed`` (64 r
 with prompts of 16 to 2,048 tokens in portions of 512), ``--long-prompt N`` (time to the
 first token of one N-token prompt in portions of 2,048), ``--sweep`` (decode at further
 batch sizes and context lengths, a line each with its share of the memory bandwidth);
-``--model 1b|70b`` and ``--batch`` change the shape.  ``--tazunex s|m`` times the Tazunex
+``--model 1b|70b`` and ``--batch`` change the shape.  ``--darovik s|m`` times the Darovik decoder
+beside the Tazunex, the Vovalix and the Llama of equal width and depth.  ``--tazunex s|m`` times the Tazunex
 decoder beside the Vovalix and the Llama of equal width and depth.  ``--vovalix s|m`` times the Vovalix
 decoder beside the Dirulorn of equal size.  ``--dirulorn s|m`` times the Dirulorn
 decoder (state-space layers beside attention-with-recurrence layers) at layer sizes of a real
@@ -144,6 +145,42 @@ TAZUNEX_SHAPES = {
     "m": {"architecture": "Tazunex", "vocab": 32000, "width": 2048, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
           "layers": _tazunex_layers(16, 2048, 32, 8, 8192, 1024)},
 }
+
+
+def _darovik_layers(n, width, heads, kv, ff, experts, top, groups, keep, window):
+    attention = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5,
+                           "mask": {"size": window}}}
+    latent = {"type": "latent_attention",
+              "mlp": {"kind": "moe", "expert": {"ff": ff // 4},
+                      "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": groups, "keep": keep}}},
+              "mixer": {"heads": 16, "dim": width // 16, "vdim": width // 16, "kv_rank": 128, "scale": 0.1}}
+    return [(attention, latent)[i % 2] for i in range(n)]
+
+
+# Darovik at the layer sizes of a real model: four copies of the stream; every other layer an
+# attention with two maps a head (maps of 64, so joint keys of 128, values of 128, windows of 1,024
+# positions) before the dense feed-forward of the Llama of the same width, the rest latent attention
+# (sixteen heads on cached rows of 128) before routed experts as the Vovalix of the same width has
+# them (four chosen ones together as wide as the dense feed-forward)
+DAROVIK_SHAPES = {
+    "s": {"architecture": "Darovik", "vocab": 32000, "width": 1024, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+          "streams": 4, "layers": _darovik_layers(8, 1024, 8, 2, 4096, 16, 4, 4, 2, 1024)},
+    "m": {"architecture": "Darovik", "vocab": 32000, "width": 2048, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+          "streams": 4, "layers": _darovik_layers(16, 2048, 16, 4, 8192, 32, 4, 8, 4, 1024)},
+}
+
+
+def bench_darovik(args) -> int:
+    """The workloads of ``bench_dirulorn`` for a Darovik shape beside the Tazunex of the same width
+    and depth (the closest model the engine has in its mixers: windowed attention and latent
+    attention), the Vovalix (routed experts) and the Llama (the dense feed-forward)."""
+    shapes = (DAROVIK_SHAPES[args.darovik], TAZUNEX_SHAPES[args.darovik], VOVALIX_SHAPES[args.darovik],
+              DIRULORN_SHAPES[args.darovik][1])
+    names = (f"darovik-{args.darovik}", f"tazunex-of-darovik-{args.darovik}", f"vovalix-of-darovik-{args.darovik}",
+             f"llama-of-darovik-{args.darovik}")
+    which = {"all": (0, 1, 2, 3), "darovik": (0,), "tazunex": (1,), "vovalix": (2,), "llama": (3,)}[args.darovik_only]
+    return _bench_design(args, shapes, names, which, args.darovik_workload)
 
 
 def bench_tazunex(args) -> int:
@@ -289,6 +326,13 @@ def parse_args():
                    help="with --dirulorn: run one of the two models only (for profiling)")
     p.add_argument("--dirulorn-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
                    help="with --dirulorn: run one of the workloads only (for profiling)")
+    p.add_argument("--darovik", default=None, choices=sorted(DAROVIK_SHAPES),
+                   help="instead of the default run: prefill and decode of the Darovik decoder at this size, and "
+                        "of the Tazunex, the Vovalix and the Llama of the same width and depth; a line each")
+    p.add_argument("--darovik-only", default="all", choices=["all", "darovik", "tazunex", "vovalix", "llama"],
+                   help="with --darovik: run one of the models only (for profiling)")
+    p.add_argument("--darovik-workload", default="all", choices=["all", "prefill", "decode8", "decode64"],
+                   help="with --darovik: run one of the workloads only (for profiling)")
     p.add_argument("--tazunex", default=None, choices=sorted(TAZUNEX_SHAPES),
                    help="time the Tazunex decoder of this size (s: 8 layers of 1,024; m: 16 of 2,048) beside "
                         "the Vovalix and the Llama of equal width and depth: prefill of 2,048 tokens, decode "
@@ -454,6 +498,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.darovik:
+        return bench_darovik(args)
     if args.tazunex:
         return bench_tazunex(args)
     if args.dirulorn:

@@ -43,6 +43,8 @@ struct SkinnyExtras {
   const float* gain;
   float* out_ss;
   int act;  // the gate's activation in the gated form (kGateSilu, kGateGeluTanh)
+  int out_act;  // the plain form: 0 stores the product (+ bias); 1 stores the square of its relu, the
+                // product rounded to bfloat16 first as if it had been stored and read again
 };
 
 // GATED: the two row tiles of a wave are rows n of the first N weight rows (gate) and rows
@@ -382,7 +384,15 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_skinny_kernel(OutT* __restrict
     for (int nt = 0; nt < NT; ++nt) {
       const int tok = nt * 16 + col;
       if (tok >= M) continue;
-      store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, acc[rt][nt] * row_scale[nt] + bv, n_left);
+      f32x4_t v = acc[rt][nt] * row_scale[nt] + bv;
+      if (ex.out_act == 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float r = fmaxf(to_float(from_float<bf16_t>(v[i])), 0.f);
+          v[i] = r * r;
+        }
+      }
+      store4<OutT>(C + static_cast<int64_t>(tok) * ldc + n_first, v, n_left);
     }
   }
 }
@@ -516,7 +526,7 @@ int check_operands(const char* who, const void* A, const void* W, int M, int N, 
   return 0;
 }
 
-const SkinnyExtras kNoExtras = {nullptr, 0, 1.f, 0.f, nullptr, 0, nullptr, nullptr, kGateSilu};
+const SkinnyExtras kNoExtras = {nullptr, 0, 1.f, 0.f, nullptr, 0, nullptr, nullptr, kGateSilu, 0};
 
 }  // namespace
 
@@ -528,6 +538,18 @@ extern "C" int kvc_gemm_skinny_silu_mul_bf16(void* C, const void* A, const void*
   return dispatch_gated(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A),
                         static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(bias), M, N, K,
                         lda, ldc, kNoExtras, packed, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int kvc_gemm_skinny_act_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
+                                        int K, int64_t lda, int64_t ldc, int act, int packed, kvc_stream stream) {
+  if (int rc = check_operands("kvc_gemm_skinny_act_bf16", A, W, M, N, K, lda, ldc, packed)) return rc;
+  if (act != 0) return kvc_fail("kvc_gemm_skinny_act_bf16: unknown activation");
+  if (M == 0) return 0;
+  SkinnyExtras ex = kNoExtras;
+  ex.out_act = 1;
+  return dispatch<bf16_t>(static_cast<bf16_t*>(C), static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W),
+                          static_cast<const bf16_t*>(bias), M, N, K, lda, ldc, ex, packed,
+                          reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M,

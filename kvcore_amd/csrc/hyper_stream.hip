@@ -26,17 +26,6 @@ namespace {
 constexpr int kMaxCopies = 8;
 
 template <int V>
-struct Vec;
-template <>
-struct Vec<1> {
-  float v[1];
-};
-template <>
-struct Vec<4> {
-  float v[4];
-};
-
-template <int V>
 __device__ __forceinline__ void ldv(const float* p, float* v) {
   if constexpr (V == 4) {
     const float4 a = *reinterpret_cast<const float4*>(p);
@@ -164,6 +153,100 @@ __global__ __launch_bounds__(256) void hyper_step_kernel(
   }
 }
 
+// The same step for rows that a block's registers hold (H <= 256 * V * NCH): every copy and the
+// sublayer's result are asked for at once, before the coefficients are looked at; the new copies
+// are stored and the sublayer input u stays in registers for the norm, so memory is read and
+// written once and the chain of dependent loads is one load long.  The sums are formed in the
+// order of the kernel above: both give the same bits.
+template <typename TY, typename TO, int C, int V, int NCH>
+__global__ __launch_bounds__(256) void hyper_step_regs_kernel(
+    TO* __restrict__ out, float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
+    const float* __restrict__ out_w, float mult, const float* __restrict__ in_w, const float* __restrict__ gain,
+    float eps, int H, int copies) {
+  __shared__ float scratch[16];
+  __shared__ float cm[C * C], co[C], ci[C];
+  float* rows = streams + static_cast<int64_t>(blockIdx.x) * copies * H;
+  const TY* yr = (y != nullptr) ? y + static_cast<int64_t>(blockIdx.x) * H : nullptr;
+  float x[NCH][C][V], yv[NCH][V];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * V;
+    if (e < H) {
+#pragma unroll
+      for (int s = 0; s < C; ++s)
+        if (s < copies) ldv<V>(rows + static_cast<int64_t>(s) * H + e, x[c][s]);
+      if (yr != nullptr) ldv<V>(yr + e, yv[c]);
+    }
+  }
+  if (threadIdx.x < C * C) {
+    const int s = threadIdx.x / C, t = threadIdx.x % C;
+    float v = (s == t) ? 1.f : 0.f;
+    if (mix != nullptr && s < copies && t < copies) v = mix[s * copies + t];
+    cm[threadIdx.x] = v;
+  }
+  if (threadIdx.x < C) {
+    const int t = threadIdx.x;
+    co[t] = (t < copies) ? mult * (out_w != nullptr ? out_w[t] : 1.f) : 0.f;
+    ci[t] = (t < copies) ? (in_w != nullptr ? in_w[t] : 1.f) : 0.f;
+  }
+  __syncthreads();
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * V;
+    if (e < H) {
+      float u[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) u[i] = 0.f;
+      if (yr != nullptr) {
+        float n[C][V];
+#pragma unroll
+        for (int t = 0; t < C; ++t) {
+          if (t < copies) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+              float acc = co[t] * yv[c][i];
+#pragma unroll
+              for (int s = 0; s < C; ++s)
+                if (s < copies) acc = fmaf(cm[s * C + t], x[c][s][i], acc);
+              n[t][i] = acc;
+            }
+            stv<V>(rows + static_cast<int64_t>(t) * H + e, n[t]);
+#pragma unroll
+            for (int i = 0; i < V; ++i) u[i] = fmaf(ci[t], n[t][i], u[i]);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < C; ++t)
+          if (t < copies) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) u[i] = fmaf(ci[t], x[c][t][i], u[i]);
+          }
+      }
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        ss += u[i] * u[i];
+        yv[c][i] = u[i];  // kept for the norm
+      }
+    }
+  }
+  if (out == nullptr) return;  // the same for the whole grid
+  const float inv = rsqrtf(block_sum(ss, scratch) / static_cast<float>(H) + eps);
+  TO* o = out + static_cast<int64_t>(blockIdx.x) * H;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e = (c * 256 + threadIdx.x) * V;
+    if (e < H) {
+      float g[V], r[V];
+      ldv<V>(gain + e, g);
+#pragma unroll
+      for (int i = 0; i < V; ++i) r[i] = g[i] * (yv[c][i] * inv);
+      stv<V>(o + e, r);
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void spread_streams_kernel(float* __restrict__ streams, const float* __restrict__ rows,
                                                              int H, int copies, int64_t n) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -177,13 +260,31 @@ template <typename TY, typename TO>
 int launch_hyper(void* out, float* streams, const void* y, const float* mix, const float* out_w, float mult,
                  const float* in_w, const float* gain, float eps, int T, int H, int copies, hipStream_t stream) {
   const bool v4 = H % 4 == 0;
+  const int chunks = (H + (v4 ? 1024 : 256) - 1) / (v4 ? 1024 : 256);  // of 256 threads x V values
 #define KVC_HYPER(C, V)                                                                                        \
   hipLaunchKernelGGL((hyper_step_kernel<TY, TO, C, V>), dim3(T), dim3(256), 0, stream, static_cast<TO*>(out), \
                      streams, static_cast<const TY*>(y), mix, out_w, mult, in_w, gain, eps, H, copies)
-  if (copies == 1) { if (v4) KVC_HYPER(1, 4); else KVC_HYPER(1, 1); }
-  else if (copies == 2) { if (v4) KVC_HYPER(2, 4); else KVC_HYPER(2, 1); }
-  else if (copies <= 4) { if (v4) KVC_HYPER(4, 4); else KVC_HYPER(4, 1); }
-  else { if (v4) KVC_HYPER(8, 4); else KVC_HYPER(8, 1); }
+#define KVC_HYPER_REGS(C, V, NCH)                                                                         \
+  hipLaunchKernelGGL((hyper_step_regs_kernel<TY, TO, C, V, NCH>), dim3(T), dim3(256), 0, stream,           \
+                     static_cast<TO*>(out), streams, static_cast<const TY*>(y), mix, out_w, mult, in_w, gain, \
+                     eps, H, copies)
+  // rows that fit the registers (up to 32 groups of V values a thread for the copies) in one pass
+#define KVC_HYPER_PICK(C)                                                      \
+  do {                                                                         \
+    if (v4 && chunks == 1) KVC_HYPER_REGS(C, 4, 1);                            \
+    else if (v4 && chunks == 2) KVC_HYPER_REGS(C, 4, 2);                       \
+    else if (v4 && chunks <= 4 && C * 4 <= 32) KVC_HYPER_REGS(C, 4, 4);        \
+    else if (v4 && chunks <= 8 && C * 8 <= 32) KVC_HYPER_REGS(C, 4, 8);        \
+    else if (!v4 && chunks <= 4) KVC_HYPER_REGS(C, 1, 4);                      \
+    else if (v4) KVC_HYPER(C, 4);                                              \
+    else KVC_HYPER(C, 1);                                                      \
+  } while (0)
+  if (copies == 1) KVC_HYPER_PICK(1);
+  else if (copies == 2) KVC_HYPER_PICK(2);
+  else if (copies <= 4) KVC_HYPER_PICK(4);
+  else KVC_HYPER_PICK(8);
+#undef KVC_HYPER_PICK
+#undef KVC_HYPER_REGS
 #undef KVC_HYPER
   return kvc_check_launch("kvc_hyper_step");
 }

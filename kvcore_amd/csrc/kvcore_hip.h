@@ -417,6 +417,11 @@ int kvc_gemm_mid_bf16(void* C, void* partial, const void* A, const void* W, cons
 int kvc_gemm_skinny_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
                          int K, int64_t lda, int64_t ldc, int out_dtype, int packed,
                          kvc_stream stream);
+// The same product with an activation on the way out, C bfloat16: act 0, the square of relu, of
+// the product (+ bias) rounded to bfloat16 first, so that it equals the product stored and
+// kvc_activation applied to it, bit for bit.
+int kvc_gemm_skinny_act_bf16(void* C, const void* A, const void* W, const void* bias, int M, int N,
+                             int K, int64_t lda, int64_t ldc, int act, int packed, kvc_stream stream);
 
 // dst = src [N, K] bfloat16 in tiles of 16 rows x 32 columns of 1 KB each, the tiles of 16
 // rows one after the other along K (N a multiple of 16, K of 64): element (n, k) goes to

@@ -94,6 +94,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, I, P],
         "kvc_gemm_f32": [P, P, P, P, I, I, I, L, L, P],
         "kvc_gemm_skinny_bf16": [P, P, P, P, I, I, I, L, L, I, I, P],
+        "kvc_gemm_skinny_act_bf16": [P, P, P, P, I, I, I, L, L, I, I, P],
         "kvc_gemm_skinny_silu_mul_bf16": [P, P, P, P, I, I, I, L, L, I, P],
         "kvc_pack_weight": [P, P, I, I, P],
         "kvc_gemm_skinny_blocks": [I, I, I, I],
@@ -1202,7 +1203,7 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
             raise KernelError("linear: a float32 result of bfloat16 operands must be contiguous")
         torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
         if bias is not None:
-            out.add_(bias.to(torch.float32))
+            out.add_(bias)  # promoted to float32 on the way, no copy of the bias
         return
     if out.dtype != torch.bfloat16:
         raise KernelError(f"linear: unsupported result type {out.dtype}")
@@ -1210,6 +1211,29 @@ def linear(out: torch.Tensor | ResidualSink, x: torch.Tensor | ScaledRows, w: to
         torch.mm(x, w.t(), out=out)
     else:
         torch.addmm(bias, x, w.t(), out=out)
+
+
+def linear_act(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, act: str) -> None:
+    """``out = act(x @ w.T (+ bias))`` with ``act`` one of :data:`ACTIVATIONS`, the product rounded
+    to the model's dtype before the activation.  Few rows of bfloat16 take the weight-streaming
+    kernel with the activation on its way out; every other shape the product and the activation
+    kernel one after the other, which gives the same bits."""
+    if act not in ACTIVATIONS:
+        raise KernelError(f"unknown activation {act!r} (known: {sorted(ACTIVATIONS)})")
+    M, K = x.shape
+    N = w.shape[0]
+    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.is_cuda
+            and M > 0 and out.shape == (M, N) and out.stride(1) == 1
+            and choose_product(M, N, K, few_rows_ok=_skinny_operands_ok(x, w), shared_rows_ok=False) == "few rows"
+            and (bias is None or (bias.dtype == torch.bfloat16 and bias.shape == (N,)))):
+        w_ptr, packed = _streamed(w)
+        _check(load().kvc_gemm_skinny_act_bf16(out.data_ptr(), x.data_ptr(), w_ptr,
+                                               None if bias is None else _dev(bias, "bias"), M, N, K, x.stride(0),
+                                               out.stride(0), ACTIVATIONS[act], packed, _stream()),
+               "kvc_gemm_skinny_act_bf16")
+        return
+    linear(out, x, w, bias)
+    activation(out, out, act)
 
 
 def choose_product(M: int, N: int, K: int, *, few_rows_ok: bool = True, shared_rows_ok: bool = True) -> str:

@@ -95,10 +95,6 @@ class DenseMLP(FeedForward):
     as stored.  ``up_name``/``down_name`` are the checkpoint's names of the two matrices relative to
     the part's prefix, ``suffix`` what follows each, ``bias_suffix`` what follows a bias."""
 
-    @property
-    def takes_scaled_rows(self) -> bool:  # x only goes into the up product
-        return self.hidden_size % 8 == 0
-
     def __init__(self, *, hidden_size: int, intermediate_size: int, activation: str = "relu_squared",
                  bias: bool = False, up_name: str = "up_proj", down_name: str = "down_proj",
                  suffix: str = ".weight", bias_suffix: str = ".bias", float32_result: bool = False) -> None:
@@ -127,8 +123,8 @@ class DenseMLP(FeedForward):
     def forward(self, x, ctx, call, sink=None):
         p, I = self.params, self.intermediate_size
         act = ctx.buf(f"mlp_act:{I}", I)
-        ops.linear(act, x, p["up_proj.weight"], p.get("up_proj.bias"))
-        ops.activation(act, act, self.activation)
+        # few rows: the product and the activation are one kernel
+        ops.linear_act(act, x, p["up_proj.weight"], p.get("up_proj.bias"), self.activation)
         if self.float32_result:
             out = ctx.buf("ffn_out_f32", self.hidden_size, torch.float32)
         else:

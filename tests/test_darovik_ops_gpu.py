@@ -106,6 +106,34 @@ def test_the_square_of_relu(dtype):
         ops.activation(out, out, "relu")
 
 
+@pytest.mark.parametrize("M,N,K,packed", [(1, 384, 256, False), (8, 1024, 512, True), (13, 200, 96, False),
+                                          (40, 512, 256, False), (300, 384, 256, False)])
+def test_product_bias_and_activation_in_one_kernel_give_the_bits_of_the_three_steps(M, N, K, packed):
+    """Few rows take the weight-streaming product with the activation on its way out; it must equal
+    the product stored in bfloat16 and the activation kernel applied to it, bit for bit, and both
+    the plain ``relu(x W^T + b)^2``."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).to(torch.bfloat16)
+    b = (torch.randn(N, generator=gen) * 0.3).to(torch.bfloat16)
+    wd = gpu(w, torch.bfloat16)
+    if packed and ops.can_pack_weight(wd):
+        ops.pack_weight(wd)
+    fused = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear_act(fused, gpu(x, torch.bfloat16), wd, gpu(b, torch.bfloat16), "relu_squared")
+    steps = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear(steps, gpu(x, torch.bfloat16), wd, gpu(b, torch.bfloat16))
+    ops.activation(steps, steps, "relu_squared")
+    assert torch.equal(fused, steps)
+    want = torch.relu(x.double() @ w.double().T + b.double()) ** 2
+    assert rel(fused, want) < 8e-3
+    f32 = torch.full((M, N), float("nan"), device=DEV)
+    ops.linear_act(f32, gpu(x.float()), gpu(w.float()), gpu(b.float()), "relu_squared")
+    assert rel(f32, want) < 2e-6
+
+
 # ------------------------------------------------------------------------- the router
 def plain_route(logits, correction, top, groups, keep, scale):
     E = logits.shape[1]
