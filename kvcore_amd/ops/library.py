@@ -44,7 +44,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_silu_mul": [P, P, I, I, I, P],
         "kvc_gate_mul": [P, P, I, I, I, I, P],
         "kvc_activation": [P, P, L, I, I, P],
-        "kvc_hyper_step": [P, I, P, P, I, P, P, F, P, P, F, I, I, I, P],
+        "kvc_hyper_step": [P, I, P, P, I, I, P, P, F, P, P, F, I, I, I, P],
         "kvc_spread_streams": [P, P, I, I, I, P],
         "kvc_diff_heads_norm": [P, P, L, F, F, F, I, I, I, I, P],
         "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, I, P],
@@ -324,18 +324,26 @@ def activation(out: torch.Tensor, x: torch.Tensor, act: str) -> None:
 HYPER_MAX_COPIES = 8
 
 
-def hyper_step(out: torch.Tensor | None, streams: torch.Tensor, copies: int, y: torch.Tensor | None = None, *,
+def hyper_step(out: torch.Tensor | None, streams: torch.Tensor, copies: int,
+               y: "torch.Tensor | SlicedRows | None" = None, *,
                mix: torch.Tensor | None = None, out_w: torch.Tensor | None = None, mult: float = 1.0,
                in_w: torch.Tensor | None = None, gain: torch.Tensor | None = None, eps: float = 0.0) -> None:
     """One step of a residual stream kept as ``copies`` rows a token (``streams [T, copies * H]``
     float32).  With ``y [T, H]``: every copy at once from the old ones, ``x_t <- sum_s mix[s, t] x_s
     + mult * out_w[t] * y`` (``mix`` None: the identity, ``out_w`` None: ones).  Then, with ``out
     [T, H]``: ``u = sum_t in_w[t] x_t`` (``in_w`` None: ones) and ``out = gain * u / sqrt(mean(u^2)
-    + eps)``.  One copy and no coefficients: ``x += mult * y`` and the norm."""
+    + eps)``.  One copy and no coefficients: ``x += mult * y`` and the norm.  ``y`` may be the
+    :class:`SlicedRows` that a product left (their sum is the result)."""
     T = streams.shape[0]
     if copies < 1 or streams.shape[1] % copies or streams.dtype != torch.float32 or not streams.is_contiguous():
         raise KernelError("hyper_step: the stream is contiguous float32 [T, copies * H]")
     H = streams.shape[1] // copies
+    slices = 1
+    if isinstance(y, SlicedRows):
+        if (y.rows, y.width) != (T, H) or y.data.dtype != torch.float32 or y.data.numel() < y.count * T * H \
+                or not y.data.is_contiguous():
+            raise KernelError("hyper_step: the partial sums do not fit")
+        slices, y = y.count, y.data.view(-1)[: T * H].view(T, H)
     for t, name in ((y, "y"), (out, "out")):
         if t is not None and (t.shape != (T, H) or not t.is_contiguous()):
             raise KernelError(f"hyper_step: {name} must be contiguous [T, H]")
@@ -346,7 +354,7 @@ def hyper_step(out: torch.Tensor | None, streams: torch.Tensor, copies: int, y: 
         raise KernelError("hyper_step: the norm needs its gain")
     _check(load().kvc_hyper_step(
         None if out is None else _dev(out, "out"), 0 if out is None else _code(out, "out"), _dev(streams, "streams"),
-        None if y is None else _dev(y, "y"), 0 if y is None else _code(y, "y"),
+        None if y is None else _dev(y, "y"), 0 if y is None else _code(y, "y"), slices,
         None if mix is None else _dev(mix, "mix"), None if out_w is None else _dev(out_w, "out_w"), float(mult),
         None if in_w is None else _dev(in_w, "in_w"), None if gain is None else _dev(gain, "gain"), float(eps),
         T, H, copies, _stream()), "kvc_hyper_step")
@@ -357,7 +365,7 @@ class StreamWrite:
     """A sublayer's result ``y [T, H]`` that has still to join a stream of ``copies`` rows a token:
     ``x_t <- sum_s mix[s, t] x_s + mult * out_w[t] * y`` (see :func:`hyper_step`)."""
 
-    y: torch.Tensor
+    y: "torch.Tensor | SlicedRows"
     copies: int
     mix: torch.Tensor | None
     out_w: torch.Tensor | None

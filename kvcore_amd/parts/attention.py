@@ -454,6 +454,10 @@ class DifferentialAttention(PagedAttention):
     any_head_size = True
     takes_sink = False  # the maps are joined between the attention and the output product's input
 
+    @property
+    def takes_slice_sink(self) -> bool:  # float32 partial sums whatever the result's type
+        return (self.heads * self.v_head_dim) % 8 == 0
+
     def __init__(self, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
                  scale: float, diff: float, eps: float, window: int = 0, page_size: int | None = None,
                  tensor_names: dict[str, str] | None = None, float32_result: bool = False,

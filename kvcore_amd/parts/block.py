@@ -294,15 +294,30 @@ class HyperConnectionBlock(Block):
         ops.stream_write_read(rows, residual, self.stream_copies, pending, in_w=in_w, gain=gain, eps=eps)
         return rows
 
+    def _slice_sink(self, part, width: int, ctx):
+        """In a step of a few dozen rows a part's last product may leave partial sums of slices
+        along K, which the kernel that carries the result into the copies adds up on its way:
+        the ``ops.SliceSink`` for that, or None where the step or the part does not take one.
+        One room serves both sublayers: a result is read before the next product is launched."""
+        if not (getattr(part, "takes_slice_sink", False) and width % 8 == 0
+                and ops.rows_sinkable(ctx.num_tokens, ctx.dtype)):
+            return None
+        return ops.SliceSink(ctx.buffers.get("block_slices", ops.mid_slices_bound(width) * ops.MID_ROWS, width,
+                                             torch.float32))
+
     def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
         if delta is not None and not isinstance(delta, ops.StreamWrite):
             raise RuntimeError("this block follows blocks of its own kind")
+        width = residual.shape[1] // self.stream_copies
         x = self._read("block_x", residual, ctx, delta, 0)
-        a = self.mixer.forward(x, ctx, call)
+        sink = self._slice_sink(self.mixer, width, ctx)
+        a = self.mixer.forward(x, ctx, call) if sink is None else self.mixer.forward(x, ctx, call, sink=sink)
         if self.mixer_only:
             return self._written(a, 0)
         x2 = self._read("block_x2", residual, ctx, self._written(a, 0), 1)
-        return self._written(self.ffn.forward(x2, ctx, call), 1)
+        sink = self._slice_sink(self.ffn, width, ctx)
+        f = self.ffn.forward(x2, ctx, call) if sink is None else self.ffn.forward(x2, ctx, call, sink=sink)
+        return self._written(f, 1)
 
     def settle(self, delta, residual: torch.Tensor, ctx) -> None:
         if delta is not None:

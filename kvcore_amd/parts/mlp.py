@@ -95,6 +95,10 @@ class DenseMLP(FeedForward):
     as stored.  ``up_name``/``down_name`` are the checkpoint's names of the two matrices relative to
     the part's prefix, ``suffix`` what follows each, ``bias_suffix`` what follows a bias."""
 
+    @property
+    def takes_slice_sink(self) -> bool:  # float32 partial sums whatever the result's type
+        return self.intermediate_size % 8 == 0
+
     def __init__(self, *, hidden_size: int, intermediate_size: int, activation: str = "relu_squared",
                  bias: bool = False, up_name: str = "up_proj", down_name: str = "down_proj",
                  suffix: str = ".weight", bias_suffix: str = ".bias", float32_result: bool = False) -> None:
@@ -125,6 +129,8 @@ class DenseMLP(FeedForward):
         act = ctx.buf(f"mlp_act:{I}", I)
         # few rows: the product and the activation are one kernel
         ops.linear_act(act, x, p["up_proj.weight"], p.get("up_proj.bias"), self.activation)
+        if sink is not None:
+            return ops.linear(sink, act, p["down_proj.weight"], p.get("down_proj.bias"))
         if self.float32_result:
             out = ctx.buf("ffn_out_f32", self.hidden_size, torch.float32)
         else:

@@ -273,7 +273,7 @@ def test_the_stream_after_every_layer_run(models, name, dtype):
         per = (got - layers[i]).pow(2).mean(1).sqrt() / layers[i].pow(2).mean(1).sqrt()
         above = int((per >= limit).sum())
         assert above <= (0 if dtype == torch.float32 else 4), f"layer run {i}: {above} tokens, worst {float(per.max()):.3e}"
-        assert float(per.median()) < limit / 3, f"layer run {i}: median {float(per.median()):.3e}"
+        assert float(per.median()) < limit / 2, f"layer run {i}: median {float(per.median()):.3e}"
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])

@@ -65,6 +65,30 @@ def test_a_sublayer_s_result_joins_the_copies_and_the_next_input_is_normed(copie
     assert rel(streams.view(T, copies, H), new) < 1e-6 and rel(out, plain.rms(new.sum(1), eps) * gain) < 2e-6
 
 
+@pytest.mark.parametrize("copies,H,slices", [(2, 96, 3), (4, 2048, 4), (1, 100, 2), (3, 5000, 2)])
+def test_a_result_left_as_partial_sums_is_added_up_on_its_way_into_the_copies(copies, H, slices):
+    """The sublayer's result as partial sums of slices, as a product cut along K leaves them."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(H + slices)
+    T, eps, mult = 29, 1e-5, 1.3
+    x = torch.randn(T, copies, H, generator=gen, dtype=F64)
+    parts = torch.randn(slices, T, H, generator=gen, dtype=F64).float().double()
+    mix = torch.eye(copies, dtype=F64) * 0.6 + 0.3 * torch.randn(copies, copies, generator=gen, dtype=F64)
+    w_in, w_out = (0.8 + 0.4 * torch.randn(copies, generator=gen, dtype=F64) for _ in range(2))
+    gain = 1 + 0.3 * torch.randn(H, generator=gen, dtype=F64)
+    new = torch.einsum("st,ksh->kth", mix, x) + mult * w_out[None, :, None] * parts.sum(0)[:, None, :]
+    want = plain.rms(torch.einsum("t,kth->kh", w_in, new), eps) * gain
+    room = torch.full((slices * T * H + 64,), float("nan"), device=DEV)
+    room[: slices * T * H] = gpu(parts).view(-1)
+    streams = gpu(x.reshape(T, copies * H))
+    out = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.stream_write_read(out, streams, copies, ops.StreamWrite(ops.SlicedRows(room, slices, T, H), copies, gpu(mix),
+                                                                gpu(w_out), mult),
+                          in_w=gpu(w_in), gain=gpu(gain), eps=eps)
+    assert rel(streams.view(T, copies, H), new) < 1e-6 and rel(out, want) < 4e-3
+
+
 def test_every_copy_starts_as_the_embedding_s_row():
     from kvcore_amd.ops import library as ops
 
