@@ -35,6 +35,7 @@ def darovik_spec(config: DarovikConfig) -> ModelSpec:
         return PartSpec("rmsnorm", {"hidden_size": H, "eps": eps, "weight_name": ""})
 
     layers: list[LayerSpec] = []
+    unread: list[str] = []  # tensors of a second sublayer that a layer without a feed-forward may still carry
     for i, layer in enumerate(config.layers):
         m = layer.mixer
         if isinstance(m, DifferentialAttentionConfig):
@@ -55,6 +56,7 @@ def darovik_spec(config: DarovikConfig) -> ModelSpec:
         if layer.mlp is None:
             ffn = PartSpec("none")
             norms = {"norm1": norm()}
+            unread += [f"l{i}.norm2", f"l{i}.hc2.in", f"l{i}.hc2.mix", f"l{i}.hc2.out"]
         elif isinstance(layer.mlp, DenseFeedForwardConfig):
             ffn = PartSpec("mlp", {
                 "hidden_size": H, "intermediate_size": layer.mlp.ff, "activation": "relu_squared", "bias": True,
@@ -80,5 +82,5 @@ def darovik_spec(config: DarovikConfig) -> ModelSpec:
         embedding=PartSpec("token_embedding", {"vocab_size": config.vocab, "hidden_size": H, "weight_name": ""}),
         head=PartSpec("linear_head", {"vocab_size": config.vocab, "hidden_size": H, "tied": True}),
         tie_word_embeddings=True, eos_token_ids=config.eos_token_ids, embed_prefix="embed",
-        final_norm_prefix="final.norm", head_prefix="head", ignored_suffixes=(),
+        final_norm_prefix="final.norm", head_prefix="head", ignored_suffixes=tuple(unread),
     )

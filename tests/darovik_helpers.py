@@ -88,7 +88,7 @@ CONFIG_D = {
         {"type": "latent_attention", "mixer": _latent(20, 16, 8, 48, 0.15), "mlp": _moe(32, 8, 2, 2.5, (4, 3))},
         {"type": "attention", "mixer": _attn(6, 2, 40, 72, 0.15, 70, 0.4), "mlp": _moe(16, 6, 2, 1.0, (6, 3))},
         {"type": "latent_attention", "mixer": _latent(2, 24, 16, 280, 0.1), "mlp": _ff(32)},
-        {"type": "attention", "mixer": _attn(3, 1, 48, 96, 0.15, 33, 0.5), "mlp": None},
+        {"type": "attention", "mixer": _attn(3, 1, 56, 112, 0.15, 33, 0.5), "mlp": None},
     ],
 }
 
