@@ -69,14 +69,28 @@ __device__ __forceinline__ void stv(bf16_t* p, const float* v) {
 
 // V values of a sublayer's result: the values themselves, or, where the product before left partial
 // sums of slices along K ([slices, T, H] float32), their sum in slice order.
+// A bias of the product that left them (one value a column, float32 or bfloat16) joins the sum last.
+struct RowBias {
+  const void* data;  // null: none
+  int dtype;         // 0 float32, 1 bfloat16
+};
+
 template <int V, typename TY>
-__device__ __forceinline__ void ld_slices(const TY* p, int slices, int64_t slice_stride, float* v) {
+__device__ __forceinline__ void ld_slices(const TY* p, int slices, int64_t slice_stride, RowBias bias, int e,
+                                          float* v) {
   ldv<V>(p, v);
   for (int s = 1; s < slices; ++s) {
     float u[V];
     ldv<V>(p + s * slice_stride, u);
 #pragma unroll
     for (int i = 0; i < V; ++i) v[i] += u[i];
+  }
+  if (bias.data != nullptr) {
+    float b[V];
+    if (bias.dtype == 0) ldv<V>(static_cast<const float*>(bias.data) + e, b);
+    else ldv<V>(static_cast<const bf16_t*>(bias.data) + e, b);
+#pragma unroll
+    for (int i = 0; i < V; ++i) v[i] += b[i];
   }
 }
 
@@ -86,7 +100,7 @@ template <typename TY, typename TO, int C, int V>
 __global__ __launch_bounds__(256) void hyper_step_kernel(
     TO* __restrict__ out, float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
     const float* __restrict__ out_w, float mult, const float* __restrict__ in_w, const float* __restrict__ gain,
-    float eps, int H, int copies, int slices, int64_t slice_stride) {
+    float eps, int H, int copies, int slices, int64_t slice_stride, RowBias bias) {
   __shared__ float scratch[16];
   __shared__ float cm[C * C], co[C], ci[C];
   if (threadIdx.x < C * C) {
@@ -111,7 +125,7 @@ __global__ __launch_bounds__(256) void hyper_step_kernel(
       if (s < copies) ldv<V>(rows + static_cast<int64_t>(s) * H + e, x[s]);
     if (yr != nullptr) {
       float yv[V];
-      ld_slices<V>(yr + e, slices, slice_stride, yv);
+      ld_slices<V>(yr + e, slices, slice_stride, bias, e, yv);
 #pragma unroll
       for (int t = 0; t < C; ++t) {
         if (t < copies) {
@@ -176,7 +190,7 @@ template <typename TY, typename TO, int C, int V, int NCH>
 __global__ __launch_bounds__(256) void hyper_step_regs_kernel(
     TO* __restrict__ out, float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
     const float* __restrict__ out_w, float mult, const float* __restrict__ in_w, const float* __restrict__ gain,
-    float eps, int H, int copies, int slices, int64_t slice_stride) {
+    float eps, int H, int copies, int slices, int64_t slice_stride, RowBias bias) {
   __shared__ float scratch[16];
   __shared__ float cm[C * C], co[C], ci[C];
   float* rows = streams + static_cast<int64_t>(blockIdx.x) * copies * H;
@@ -189,7 +203,7 @@ __global__ __launch_bounds__(256) void hyper_step_regs_kernel(
 #pragma unroll
       for (int s = 0; s < C; ++s)
         if (s < copies) ldv<V>(rows + static_cast<int64_t>(s) * H + e, x[c][s]);
-      if (yr != nullptr) ld_slices<V>(yr + e, slices, slice_stride, yv[c]);
+      if (yr != nullptr) ld_slices<V>(yr + e, slices, slice_stride, bias, e, yv[c]);
     }
   }
   if (threadIdx.x < C * C) {
@@ -273,18 +287,18 @@ __global__ __launch_bounds__(256) void spread_streams_kernel(float* __restrict__
 template <typename TY, typename TO>
 int launch_hyper(void* out, float* streams, const void* y, const float* mix, const float* out_w, float mult,
                  const float* in_w, const float* gain, float eps, int T, int H, int copies, int slices,
-                 hipStream_t stream) {
+                 RowBias bias, hipStream_t stream) {
   const int64_t slice_stride = static_cast<int64_t>(T) * H;
   const bool v4 = H % 4 == 0;
   const int chunks = (H + (v4 ? 1024 : 256) - 1) / (v4 ? 1024 : 256);  // of 256 threads x V values
 #define KVC_HYPER(C, V)                                                                                        \
   hipLaunchKernelGGL((hyper_step_kernel<TY, TO, C, V>), dim3(T), dim3(256), 0, stream, static_cast<TO*>(out), \
                      streams, static_cast<const TY*>(y), mix, out_w, mult, in_w, gain, eps, H, copies, \
-                     slices, slice_stride)
+                     slices, slice_stride, bias)
 #define KVC_HYPER_REGS(C, V, NCH)                                                                         \
   hipLaunchKernelGGL((hyper_step_regs_kernel<TY, TO, C, V, NCH>), dim3(T), dim3(256), 0, stream,           \
                      static_cast<TO*>(out), streams, static_cast<const TY*>(y), mix, out_w, mult, in_w, gain, \
-                     eps, H, copies, slices, slice_stride)
+                     eps, H, copies, slices, slice_stride, bias)
   // rows that fit the registers (up to 32 groups of V values a thread for the copies) in one pass
 #define KVC_HYPER_PICK(C)                                                      \
   do {                                                                         \
@@ -309,12 +323,15 @@ int launch_hyper(void* out, float* streams, const void* y, const float* mix, con
 }  // namespace
 
 extern "C" int kvc_hyper_step(void* out, int out_dtype, float* streams, const void* y, int y_dtype, int y_slices,
-                              const float* mix, const float* out_w, float mult, const float* in_w, const float* gain,
+                              const void* y_bias, int y_bias_dtype, const float* mix, const float* out_w, float mult, const float* in_w, const float* gain,
                               float eps, int T, int H, int copies, kvc_stream stream) {
   if (T < 0 || H <= 0 || copies < 1 || copies > kMaxCopies)
     return kvc_fail("kvc_hyper_step: bad sizes (one to eight copies of the stream)");
   if (streams == nullptr) return kvc_fail("kvc_hyper_step: null stream");
   if (y_slices < 1 || (y_slices > 1 && y_dtype != 0)) return kvc_fail("kvc_hyper_step: partial sums are float32");
+  if (y_bias != nullptr && (y == nullptr || (y_bias_dtype != 0 && y_bias_dtype != 1)))
+    return kvc_fail("kvc_hyper_step: a bias comes with a result and is float32 or bfloat16");
+  const RowBias bias{y_bias, y_bias_dtype};
   if (out != nullptr && gain == nullptr) return kvc_fail("kvc_hyper_step: the norm needs its gain");
   if (out == nullptr && y == nullptr) return 0;  // nothing to do
   if (T == 0) return 0;
@@ -324,12 +341,12 @@ extern "C" int kvc_hyper_step(void* out, int out_dtype, float* streams, const vo
     return kvc_fail("kvc_hyper_step: unknown dtype code");
   hipStream_t st = S(stream);
   if (y_dtype == 0 && out_dtype == 0)
-    return launch_hyper<float, float>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, st);
+    return launch_hyper<float, float>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, bias, st);
   if (y_dtype == 0)
-    return launch_hyper<float, bf16_t>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, st);
+    return launch_hyper<float, bf16_t>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, bias, st);
   if (out_dtype == 0)
-    return launch_hyper<bf16_t, float>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, st);
-  return launch_hyper<bf16_t, bf16_t>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, st);
+    return launch_hyper<bf16_t, float>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, bias, st);
+  return launch_hyper<bf16_t, bf16_t>(out, streams, y, mix, out_w, mult, in_w, gain, eps, T, H, copies, y_slices, bias, st);
 }
 
 extern "C" int kvc_spread_streams(float* streams, const float* rows, int T, int H, int copies, kvc_stream stream) {

@@ -382,11 +382,12 @@ int kvc_head_gate(void* out, const void* x, int64_t x_stride, const void* gate, 
                   int T, int heads, int head_stride, int skip, int n, int dtype, kvc_stream stream);
 
 // A residual stream of `copies` (1 to 8) rows a token, streams [T, copies, H] float32.  With y ([T, H]
-// of y_dtype; or, y_slices > 1, that many float32 partial sums [y_slices, T, H] whose sum it is): x_t <- sum_s mix[s * copies + t] x_s + mult * out_w[t] * y for all copies at once (mix
+// of y_dtype; or, y_slices > 1, that many float32 partial sums [y_slices, T, H] whose sum it is; plus
+// y_bias [H] of y_bias_dtype, if not null): x_t <- sum_s mix[s * copies + t] x_s + mult * out_w[t] * y for all copies at once (mix
 // null: the identity, out_w null: ones).  Then, with out ([T, H] of out_dtype): u = sum_t in_w[t] x_t
 // (in_w null: ones), out = gain * u / sqrt(mean(u^2) + eps).
 int kvc_hyper_step(void* out, int out_dtype, float* streams, const void* y, int y_dtype, int y_slices,
-                   const float* mix, const float* out_w, float mult, const float* in_w, const float* gain, float eps,
+                   const void* y_bias, int y_bias_dtype, const float* mix, const float* out_w, float mult, const float* in_w, const float* gain, float eps,
                    int T, int H, int copies, kvc_stream stream);
 // streams[t, c, :] = rows[t, :] for every copy c.
 int kvc_spread_streams(float* streams, const float* rows, int T, int H, int copies, kvc_stream stream);

@@ -44,7 +44,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_silu_mul": [P, P, I, I, I, P],
         "kvc_gate_mul": [P, P, I, I, I, I, P],
         "kvc_activation": [P, P, L, I, I, P],
-        "kvc_hyper_step": [P, I, P, P, I, I, P, P, F, P, P, F, I, I, I, P],
+        "kvc_hyper_step": [P, I, P, P, I, I, P, I, P, P, F, P, P, F, I, I, I, P],
         "kvc_spread_streams": [P, P, I, I, I, P],
         "kvc_diff_heads_norm": [P, P, L, F, F, F, I, I, I, I, P],
         "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, I, P],
@@ -338,12 +338,14 @@ def hyper_step(out: torch.Tensor | None, streams: torch.Tensor, copies: int,
     if copies < 1 or streams.shape[1] % copies or streams.dtype != torch.float32 or not streams.is_contiguous():
         raise KernelError("hyper_step: the stream is contiguous float32 [T, copies * H]")
     H = streams.shape[1] // copies
-    slices = 1
+    slices, bias = 1, None
     if isinstance(y, SlicedRows):
         if (y.rows, y.width) != (T, H) or y.data.dtype != torch.float32 or y.data.numel() < y.count * T * H \
                 or not y.data.is_contiguous():
             raise KernelError("hyper_step: the partial sums do not fit")
-        slices, y = y.count, y.data.view(-1)[: T * H].view(T, H)
+        if y.bias is not None and (y.bias.shape != (H,) or not y.bias.is_contiguous()):
+            raise KernelError("hyper_step: the bias does not fit")
+        slices, bias, y = y.count, y.bias, y.data.view(-1)[: T * H].view(T, H)
     for t, name in ((y, "y"), (out, "out")):
         if t is not None and (t.shape != (T, H) or not t.is_contiguous()):
             raise KernelError(f"hyper_step: {name} must be contiguous [T, H]")
@@ -355,6 +357,7 @@ def hyper_step(out: torch.Tensor | None, streams: torch.Tensor, copies: int,
     _check(load().kvc_hyper_step(
         None if out is None else _dev(out, "out"), 0 if out is None else _code(out, "out"), _dev(streams, "streams"),
         None if y is None else _dev(y, "y"), 0 if y is None else _code(y, "y"), slices,
+        None if bias is None else _dev(bias, "bias"), 0 if bias is None else _code(bias, "bias"),
         None if mix is None else _dev(mix, "mix"), None if out_w is None else _dev(out_w, "out_w"), float(mult),
         None if in_w is None else _dev(in_w, "in_w"), None if gain is None else _dev(gain, "gain"), float(eps),
         T, H, copies, _stream()), "kvc_hyper_step")
@@ -884,20 +887,25 @@ class SliceSink:
     """Where the last product of a part goes when the block behind it norms the result before
     it joins the stream (steps of 17 to 192 rows): ``slices`` is float32 room for the partial
     sums of a product cut along K (``mid_slices_bound(N) * T * N`` values).  ``linear`` leaves
-    them there and returns :class:`SlicedRows`; ``norm_add_norm`` sums them on its way."""
+    them there and returns :class:`SlicedRows`; ``norm_add_norm`` sums them on its way.
+    ``takes_bias``: the consumer adds a product's bias itself (``SlicedRows.bias``), so a product
+    with a bias may be cut along K as well."""
 
     slices: torch.Tensor
+    takes_bias: bool = False
 
 
 @dataclass
 class SlicedRows:
     """``count`` partial sums ``[count, T, N]`` float32 at the start of ``data``'s storage: rows
-    of a product that the consumer adds up (one slice is the product itself)."""
+    of a product that the consumer adds up (one slice is the product itself).  ``bias``: the
+    product's bias ``[N]``, still to be added to the sum (only for a sink that ``takes_bias``)."""
 
     data: torch.Tensor
     count: int
     rows: int
     width: int
+    bias: torch.Tensor | None = None
 
 
 # The most rows the kernel that shares its rows through LDS takes (twelve tiles of 16 a wave).
@@ -1117,13 +1125,14 @@ def _slices_mid(sink: SliceSink, x: torch.Tensor, w: torch.Tensor, bias: torch.T
     N = w.shape[0]
     if sink.slices.dtype != torch.float32 or not sink.slices.is_contiguous():
         raise KernelError("linear: the room for partial sums must be contiguous float32")
-    ours = (N < 8192 or K > 8192) and mid_rows_ok(M, bool(_streamed(w, N)[1]), MID_ROWS) and bias is None
+    ours = (N < 8192 or K > 8192) and mid_rows_ok(M, bool(_streamed(w, N)[1]), MID_ROWS) \
+        and (bias is None or (sink.takes_bias and bias.shape == (N,) and bias.is_contiguous()))
     if ours and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and mid_operands_ok(x, w) and N % 8 == 0:
         slices = mid_slices(N, K)
         if sink.slices.numel() < slices * M * N:
             raise KernelError("linear: the room for partial sums is too small")
         gemm_mid(None, x, w, mode=2, partial=sink.slices)
-        return SlicedRows(sink.slices, slices, M, N)
+        return SlicedRows(sink.slices, slices, M, N, bias)
     if sink.slices.numel() < M * N:
         raise KernelError("linear: the room for partial sums is too small")
     linear(sink.slices.view(-1)[: M * N].view(M, N), x, w, bias)
@@ -1605,6 +1614,8 @@ def norm_add_norm(out: torch.Tensor | None, residual: torch.Tensor, delta: "torc
     T, H = residual.shape
     slices = 1
     if isinstance(delta, SlicedRows):
+        if delta.bias is not None:
+            raise KernelError("norm_add_norm: partial sums whose bias is still to be added")
         if (delta.rows, delta.width) != (T, H) or delta.data.dtype != torch.float32 \
                 or delta.data.numel() < delta.count * T * H or not delta.data.is_contiguous():
             raise KernelError("norm_add_norm: the partial sums do not fit")

@@ -303,7 +303,7 @@ class HyperConnectionBlock(Block):
                 and ops.rows_sinkable(ctx.num_tokens, ctx.dtype)):
             return None
         return ops.SliceSink(ctx.buffers.get("block_slices", ops.mid_slices_bound(width) * ops.MID_ROWS, width,
-                                             torch.float32))
+                                             torch.float32), takes_bias=True)
 
     def forward(self, delta, residual: torch.Tensor, ctx, call, next_block=None):
         if delta is not None and not isinstance(delta, ops.StreamWrite):

@@ -77,16 +77,50 @@ def test_a_result_left_as_partial_sums_is_added_up_on_its_way_into_the_copies(co
     mix = torch.eye(copies, dtype=F64) * 0.6 + 0.3 * torch.randn(copies, copies, generator=gen, dtype=F64)
     w_in, w_out = (0.8 + 0.4 * torch.randn(copies, generator=gen, dtype=F64) for _ in range(2))
     gain = 1 + 0.3 * torch.randn(H, generator=gen, dtype=F64)
-    new = torch.einsum("st,ksh->kth", mix, x) + mult * w_out[None, :, None] * parts.sum(0)[:, None, :]
-    want = plain.rms(torch.einsum("t,kth->kh", w_in, new), eps) * gain
     room = torch.full((slices * T * H + 64,), float("nan"), device=DEV)
     room[: slices * T * H] = gpu(parts).view(-1)
-    streams = gpu(x.reshape(T, copies * H))
-    out = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops.stream_write_read(out, streams, copies, ops.StreamWrite(ops.SlicedRows(room, slices, T, H), copies, gpu(mix),
-                                                                gpu(w_out), mult),
-                          in_w=gpu(w_in), gain=gpu(gain), eps=eps)
-    assert rel(streams.view(T, copies, H), new) < 1e-6 and rel(out, want) < 4e-3
+    # without a bias, and with the product's bias still to be added (in either dtype)
+    for bias_dtype in (None, torch.float32, torch.bfloat16):
+        bias = None if bias_dtype is None else torch.randn(H, generator=gen, dtype=F64).to(bias_dtype).double()
+        y = parts.sum(0) + (0 if bias is None else bias)
+        new = torch.einsum("st,ksh->kth", mix, x) + mult * w_out[None, :, None] * y[:, None, :]
+        want = plain.rms(torch.einsum("t,kth->kh", w_in, new), eps) * gain
+        streams = gpu(x.reshape(T, copies * H))
+        out = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+        rows = ops.SlicedRows(room, slices, T, H, None if bias is None else gpu(bias, bias_dtype))
+        ops.stream_write_read(out, streams, copies, ops.StreamWrite(rows, copies, gpu(mix), gpu(w_out), mult),
+                              in_w=gpu(w_in), gain=gpu(gain), eps=eps)
+        assert rel(streams.view(T, copies, H), new) < 1e-6 and rel(out, want) < 4e-3
+
+
+@pytest.mark.parametrize("M,N,K,packed", [(40, 1024, 2048, True), (64, 512, 4096, True), (23, 96, 80, False),
+                                          (100, 2048, 8192, True), (33, 192, 512, False)])
+def test_a_product_with_a_bias_that_leaves_partial_sums_for_the_stream(M, N, K, packed):
+    """``linear`` into a ``SliceSink`` that takes the bias along, and the stream kernel that adds the
+    slices and the bias up, against the plain product on the same rounded operands: shapes that the
+    weight-streaming kernel cuts along K, and shapes it does not take."""
+    from kvcore_amd.ops import library as ops
+
+    gen = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=gen) * K ** -0.5).to(torch.bfloat16)
+    b = torch.randn(N, generator=gen).to(torch.bfloat16)
+    x = torch.randn(M, 2, N, generator=gen, dtype=F64)
+    wd = gpu(w, torch.bfloat16)
+    if packed and ops.can_pack_weight(wd):
+        ops.pack_weight(wd)
+    room = torch.full((ops.mid_slices_bound(N) * ops.MID_ROWS * N,), float("nan"), device=DEV)
+    got = ops.linear(ops.SliceSink(room, takes_bias=True), gpu(a, torch.bfloat16), wd, gpu(b, torch.bfloat16))
+    assert isinstance(got, ops.SlicedRows) and (got.rows, got.width) == (M, N)
+    if packed and K % 512 == 0 and ops.can_pack_weight(wd):
+        assert got.count == ops.mid_slices(N, K) and got.bias is not None
+    streams = gpu(x.reshape(M, 2 * N))
+    ops.stream_write_read(None, streams, 2, ops.StreamWrite(got, 2, None, None, 0.5))
+    want = x + 0.5 * (a.double() @ w.double().T + b.double())[:, None, :]
+    assert rel(streams.view(M, 2, N), want) < 1e-5
+    # a sink that does not take the bias gets it added by the product, as one slice
+    got = ops.linear(ops.SliceSink(room), gpu(a, torch.bfloat16), wd, gpu(b, torch.bfloat16))
+    assert got.bias is None and got.count == 1
 
 
 def test_every_copy_starts_as_the_embedding_s_row():
