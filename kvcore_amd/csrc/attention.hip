@@ -50,7 +50,8 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
     const T* __restrict__ v_cache, const int32_t* __restrict__ table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_req,
     const int32_t* __restrict__ slots, int nh, int nkv, int d, int dv, int page_size, int num_pages,
-    float scale, int window, const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks) {
+    float scale, int window, const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks,
+    int out_f32) {
   __shared__ float q_s[kWavesPerBlock][MAXD];
   __shared__ float p_s[kWavesPerBlock][kWave];
   __shared__ int64_t off_s[kWavesPerBlock][kWave];   // K row of each key of the tile
@@ -62,12 +63,17 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
   const int h_raw = blockIdx.y * kWavesPerBlock + wave;
   const bool head_live = h_raw < nh;
   const int h = head_live ? h_raw : nh - 1;
+  // the results in the operands' type, or (out_f32) as the float32 sums they are
   T* o = out + (static_cast<int64_t>(t) * nh + h) * dv;
+  float* o32 = reinterpret_cast<float*>(out) + (static_cast<int64_t>(t) * nh + h) * dv;
 
   const int req = token_req[t];
   if (req < 0) {  // padding token: the whole block takes this branch
     if (head_live)
-      for (int i = lane; i < dv; i += kWave) o[i] = from_float<T>(0.f);
+      for (int i = lane; i < dv; i += kWave) {
+        if (out_f32) o32[i] = 0.f;
+        else o[i] = from_float<T>(0.f);
+      }
     return;
   }
   const int pos = positions[t];
@@ -157,7 +163,10 @@ __global__ __launch_bounds__(kWavesPerBlock* kWave) void paged_attention_wave_ke
 #pragma unroll
   for (int i = 0; i < MAXD / kWave; ++i) {
     const int e = lane + i * kWave;
-    if (e < dv) o[e] = from_float<T>(acc[i] * inv);
+    if (e < dv) {
+      if (out_f32) o32[e] = acc[i] * inv;
+      else o[e] = from_float<T>(acc[i] * inv);
+    }
   }
 }
 
@@ -168,7 +177,7 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                                    const int32_t* positions, const int32_t* token_req,
                                    const int32_t* slots, int T, int nh, int nkv, int d, int dv,
                                    int page_size, int num_pages, float scale, int window,
-                                   const float* slopes, int chunk, const float* sinks, int dtype,
+                                   const float* slopes, int chunk, const float* sinks, int out_f32, int dtype,
                                    kvc_stream stream) {
   if (T < 0 || nh <= 0 || nkv <= 0 || page_size <= 0 || num_pages <= 0 || table_stride <= 0)
     return kvc_fail("kvc_paged_attention: bad sizes");
@@ -189,7 +198,7 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                            static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
                            static_cast<const Tp*>(v_cache), table, table_stride, positions,
                            token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window, slopes,
-                           chunk, sinks));
+                           chunk, sinks, out_f32));
     return kvc_check_launch("kvc_paged_attention");
   }
   KVC_DISPATCH_DTYPE(
@@ -199,7 +208,7 @@ extern "C" int kvc_paged_attention(void* out, const void* q, int64_t q_stride, c
                          static_cast<const Tp*>(q), q_stride, static_cast<const Tp*>(k_cache),
                          static_cast<const Tp*>(v_cache), table, table_stride, positions,
                          token_req, slots, nh, nkv, d, dv, page_size, num_pages, scale, window, slopes,
-                         chunk, sinks));
+                         chunk, sinks, out_f32));
   return kvc_check_launch("kvc_paged_attention");
 }
 

@@ -49,6 +49,7 @@ constexpr size_t kLdsLimit = 64 * 1024;
 
 struct DecodeArgs {
   bf16_t* out;
+  int out_f32;  // out receives float32 values (the sums as they are) instead of bfloat16
   float* part_o;
   float* part_ml;
   const bf16_t* qkv;  // rows [nh q heads | nkv k heads | nkv v heads] of d
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
   if (trow_idx < 0) {  // padding token
     if (nsplit == 1) {
       for (int idx = tid; idx < g * D; idx += nthreads)
-        a.out[(static_cast<int64_t>(t) * nh + hk * g) * D + idx] = from_float<bf16_t>(0.f);
+        store_result(a.out, (static_cast<int64_t>(t) * nh + hk * g) * D + idx, 0.f, a.out_f32);
     } else if (tid < g) {
       float* ml = a.part_ml + ((static_cast<int64_t>(t) * nh + hk * g + tid) * nsplit + split) * 2;
       ml[0] = -INFINITY;
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
     }
     const int64_t th = static_cast<int64_t>(t) * nh + hk * g + h;
     if (nsplit == 1) {
-      a.out[th * D + e] = from_float<bf16_t>(denom > 0.f ? acc / denom : 0.f);
+      store_result(a.out, th * D + e, denom > 0.f ? acc / denom : 0.f, a.out_f32);
     } else {
       a.part_o[(th * nsplit + split) * D + e] = acc;
       if (e == 0) {
@@ -417,7 +418,7 @@ __global__ __launch_bounds__(max_waves<D>() * 64) void decode_attention_kernel(c
 // another wave; the partial outputs are asked for before the weights are known.
 constexpr int kMaxSplits = kMaxAttentionSplits;
 __global__ void decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
-                                      const float* __restrict__ part_ml, int D, int nsplit) {
+                                      const float* __restrict__ part_ml, int D, int nsplit, int out_f32) {
   const int64_t th = blockIdx.x;  // token * nh + head
   const int lane = threadIdx.x & 63;
   const float* ml = part_ml + th * nsplit * 2;
@@ -446,7 +447,7 @@ __global__ void decode_combine_kernel(bf16_t* __restrict__ out, const float* __r
         if (s0 + i < nsplit && w > 0.f) acc += w * v[i];
       }
     }
-    if (live) out[th * D + e] = from_float<bf16_t>(denom > 0.f ? acc / denom : 0.f);
+    if (live) store_result(out, th * D + e, denom > 0.f ? acc / denom : 0.f, out_f32);
   }
 }
 
@@ -473,19 +474,19 @@ int launch_decode(DecodeArgs& args, int T, hipStream_t stream) {
                      lds_total(waves, g, D, args.lds_pages), stream, args);
   if (args.nsplit > 1)
     hipLaunchKernelGGL(decode_combine_kernel, dim3(T * args.nh), dim3((D + 63) / 64 * 64), 0, stream,
-                       args.out, args.part_o, args.part_ml, D, args.nsplit);
+                       args.out, args.part_o, args.part_ml, D, args.nsplit, args.out_f32);
   return kvc_check_launch("kvc_decode_attention");
 }
 
 }  // namespace
 
 int kvc::launch_attention_combine(bf16_t* out, const float* part_o, const float* part_ml, int64_t rows,
-                                  int d, int nsplit, hipStream_t stream) {
+                                  int d, int nsplit, int out_f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (rows > 0x7fffffff || nsplit < 1 || nsplit > kMaxAttentionSplits)
     return kvc_fail("attention combine: bad sizes");
   hipLaunchKernelGGL(decode_combine_kernel, dim3(static_cast<unsigned>(rows)), dim3((d + 63) / 64 * 64), 0,
-                     stream, out, part_o, part_ml, d, nsplit);
+                     stream, out, part_o, part_ml, d, nsplit, out_f32);
   return kvc_check_launch("attention combine");
 }
 
@@ -517,7 +518,7 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
                                     const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T, int nh,
                                     int nkv, int d, int page_size, int num_pages, float scale,
                                     int window, const float* slopes, int chunk, const float* sinks,
-                                    int nsplit, kvc_stream stream) {
+                                    int nsplit, int out_f32, kvc_stream stream) {
   if (!kvc_decode_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_decode_attention: unsupported shape (bfloat16, head size a multiple of 32 "
                     "up to 256, at most 16 query heads per kv head, page size a multiple of 16)");
@@ -534,6 +535,7 @@ extern "C" int kvc_decode_attention(void* out, void* part_o, void* part_ml, cons
   if (T == 0) return 0;
   DecodeArgs args;
   args.out = static_cast<bf16_t*>(out);
+  args.out_f32 = out_f32;
   args.part_o = static_cast<float*>(part_o);
   args.part_ml = static_cast<float*>(part_ml);
   args.qkv = static_cast<const bf16_t*>(qkv);

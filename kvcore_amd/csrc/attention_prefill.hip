@@ -86,7 +86,8 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
     int nkv, int page_size, int num_pages, float scale_log2e, int window,
     const float* __restrict__ slopes, int chunk, const float* __restrict__ sinks, float* __restrict__ part_o,
     float* __restrict__ part_ml, int single,
-    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim, int interleaved) {
+    const float* __restrict__ cos_tab, const float* __restrict__ sin_tab, int rot_dim, int interleaved,
+    int out_f32) {
   constexpr int kKeyBlocks = KB;
   constexpr int NJ = D / 16;
   constexpr int NC = D / 32;
@@ -633,7 +634,14 @@ __global__ __launch_bounds__(W * 64, (W == 4) ? 2 : 1) void prefill_attention_ke
       continue;
     }
     const float inv = (l_row > 0.f) ? 1.f / l_row : 0.f;
-    bf16_t* op = out + (static_cast<int64_t>(my_tok[ct]) * nh + my_head[ct]) * D + 4 * quad;
+    const int64_t at = (static_cast<int64_t>(my_tok[ct]) * nh + my_head[ct]) * D + 4 * quad;
+    if (out_f32) {  // the sums as they are, for a consumer that joins them before anything is rounded
+      float* op = reinterpret_cast<float*>(out) + at;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) *reinterpret_cast<f32x4_t*>(op + 16 * j) = o_acc[ct][j] * inv;
+      continue;
+    }
+    bf16_t* op = out + at;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const f32x4_t v = o_acc[ct][j] * inv;
@@ -651,7 +659,7 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
                       int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
                       const float* slopes, int chunk, const float* sinks, float* part_o, float* part_ml, int nsplit, int single,
                       const float* cos_tab,
-                      const float* sin_tab, int rot_dim, int interleaved, hipStream_t stream) {
+                      const float* sin_tab, int rot_dim, int interleaved, int out_f32, hipStream_t stream) {
   const int g = nh / nkv;
   const int bq = (16 * W * CT) / g;
   // every request may end in a ragged tile and have an odd number of tiles
@@ -678,8 +686,9 @@ int launch_prefill_ct(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16
   hipLaunchKernelGGL((prefill_attention_kernel<D, CT, KB, W>), dim3(static_cast<unsigned>(wide), 1, nsplit), dim3(W * 64),
                      lds_bytes, stream, out, q, q_stride, k_cache, v_cache, table, table_stride, positions,
                      q_start, slots, R, nh, nkv, page_size, num_pages, scale * kLog2e, window, slopes, chunk,
-                     sinks, part_o, part_ml, single, cos_tab, sin_tab, rot_dim, interleaved);
-  if (nsplit > 1) return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, stream);
+                     sinks, part_o, part_ml, single, cos_tab, sin_tab, rot_dim, interleaved, out_f32);
+  if (nsplit > 1)
+    return launch_attention_combine(out, part_o, part_ml, static_cast<int64_t>(T) * nh, D, nsplit, out_f32, stream);
   return kvc_check_launch("kvc_prefill_attention");
 }
 
@@ -690,7 +699,7 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
                    int R, int nh, int nkv, int page_size, int num_pages, float scale, int window,
                    const float* slopes, int chunk, const float* sinks, float* part_o, float* part_ml, int nsplit,
                    const float* cos_tab, const float* sin_tab,
-                   int rot_dim, int interleaved, hipStream_t stream) {
+                   int rot_dim, int interleaved, int out_f32, hipStream_t stream) {
   const int g = nh / nkv;
   // Blocks of four waves lie two to a compute unit, blocks of eight waves one.  Tiles of 64
   // query rows, two a block one after the other (a late and an early one), are the fastest as
@@ -748,7 +757,7 @@ int launch_prefill(bf16_t* out, const bf16_t* q, int64_t q_stride, const bf16_t*
   return launch_prefill_ct<D, CT_, W_>(out, q, q_stride, k_cache, v_cache, table, table_stride, positions, \
                                        q_start, slots, T, R, nh, nkv, page_size, num_pages, scale, window, \
                                        slopes, chunk, sinks, part_o, part_ml, nsplit, single, cos_tab, sin_tab, rot_dim,     \
-                                       interleaved, stream)
+                                       interleaved, out_f32, stream)
   if (waves == 8) {
     if (ct == 2) KVC_LAUNCH_PREFILL(2, 8);
     KVC_LAUNCH_PREFILL(1, 8);
@@ -774,7 +783,7 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
                                      const int32_t* slots, int T, int R, int nh, int nkv, int d,
                                      int page_size, int num_pages, float scale, int window,
                                      const float* slopes, int chunk, const float* sinks, void* part_o, void* part_ml, int nsplit, const float* cos_tab,
-                                     const float* sin_tab, int rot_dim, int interleaved,
+                                     const float* sin_tab, int rot_dim, int interleaved, int out_f32,
                                      kvc_stream stream) {
   if (!kvc_prefill_attention_supported(nh, nkv, d, page_size, 1))
     return kvc_fail("kvc_prefill_attention: unsupported shape (bfloat16, head size 64 or 128, at "
@@ -803,8 +812,9 @@ extern "C" int kvc_prefill_attention(void* out, const void* q, int64_t q_stride,
   if (d == 64)
     return launch_prefill<64>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                               positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                              window, slopes, chunk, sinks, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
+                              window, slopes, chunk, sinks, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, out_f32, s);
   return launch_prefill<128>(static_cast<bf16_t*>(out), qq, q_stride, kc, vc, table, table_stride,
                              positions, q_start, slots, T, R, nh, nkv, page_size, num_pages, scale,
-                             window, slopes, chunk, sinks, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved, s);
+                             window, slopes, chunk, sinks, po, pml, nsplit, cos_tab, sin_tab, rot_dim, interleaved,
+                             out_f32, s);
 }

@@ -127,12 +127,14 @@ int kvc_rope_kv_write(void* qkv, void* k_cache, void* v_cache, const float* cos_
 // h.  chunk > 0: a token sees only the keys j with j / chunk == p / chunk.  sinks (float32 [nh],
 // or null): exp(sinks[h]) is added to the softmax's denominator of head h: a logit of its own,
 // taken as it is (scale does not apply), that brings no value into the weighted sum.
+// out_f32: out is float32 whatever dtype says of the operands (the weighted sums as they are, for a
+// consumer that joins results before anything is rounded); the two kernels below take it too.
 int kvc_paged_attention(void* out, const void* q, int64_t q_stride, const void* k_cache,
                         const void* v_cache, const int32_t* table, int table_stride,
                         const int32_t* positions, const int32_t* token_req,
                         const int32_t* slots, int T, int nh, int nkv, int d, int dv, int page_size,
                         int num_pages, float scale, int window, const float* slopes, int chunk,
-                        const float* sinks, int dtype, kvc_stream stream);
+                        const float* sinks, int out_f32, int dtype, kvc_stream stream);
 
 // What kvc_rope_kv_write does, for heads whose keys (d) and values (dv) may differ in size,
 // with a norm of every q and k head before the rotation: rows of qkv are [nh q heads of d |
@@ -329,7 +331,7 @@ int kvc_decode_attention(void* out, void* part_o, void* part_ml, const void* qkv
                          const float* sin_tab, int rot_dim, int interleaved, int write_kv, int T,
                          int nh, int nkv, int d, int page_size, int num_pages, float scale,
                          int window, const float* slopes, int chunk, const float* sinks, int nsplit,
-                         kvc_stream stream);
+                         int out_f32, kvc_stream stream);
 
 // The same attention for bfloat16 portions of prompts on the matrix cores: a block per
 // (tile of a request's tokens, kv head), keys staged through LDS.  q_start [R+1] bounds
@@ -348,7 +350,7 @@ int kvc_prefill_attention(void* out, const void* q, int64_t q_stride, const void
                           float scale, int window, const float* slopes, int chunk, const float* sinks, void* part_o,
                           void* part_ml, int nsplit,
                           const float* cos_tab, const float* sin_tab, int rot_dim, int interleaved,
-                          kvc_stream stream);
+                          int out_f32, kvc_stream stream);
 
 // ---- norms after a sublayer, norms over a whole projection, gates per head (norm_ops.hip)
 // residual[t, :] += post_gain * delta[t, :] / sqrt(mean(delta[t, :]^2) + eps), and then, if out is
@@ -361,9 +363,10 @@ int kvc_norm_add_norm(void* out, int out_dtype, float* residual, const void* del
                       const float* post_gain, float eps, const float* next_gain, float next_eps,
                       int T, int H, int slices, kvc_stream stream);
 // Rows of attn are [heads][2][dv]: out[t, h] = (a1 - lambda * a2) / sqrt(mean((a1 - lambda * a2)^2) + eps)
-// * post over the head's dv values, out [T, heads * dv]; float32 arithmetic.
-int kvc_diff_heads_norm(void* out, const void* attn, int64_t attn_stride, float lambda, float eps, float post,
-                        int T, int heads, int dv, int dtype, kvc_stream stream);
+// * post over the head's dv values, out [T, heads * dv] of dtype; attn of attn_dtype (dtype, or float32);
+// float32 arithmetic.
+int kvc_diff_heads_norm(void* out, const void* attn, int64_t attn_stride, int attn_dtype, float lambda, float eps,
+                        float post, int T, int heads, int dv, int dtype, kvc_stream stream);
 // Rows of qkv are [nq | nk | ...]: the first nq values (all query heads at once) are divided by
 // their root mean square (eps inside the root) and multiplied by q_gain [nq], the next nk values
 // likewise with k_gain [nk], in place; with copy_k the nk values as they were before the norm

@@ -256,8 +256,8 @@ __global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ out, con
 // Two softmax maps a head over the same values: rows of attn are [heads][2][dv]; the second map is
 // taken off the first lambda times, the difference divided by its root mean square over the
 // head's dv values (eps inside the root, no gain) and multiplied by post.  A wave a (token, head).
-template <typename T>
-__global__ __launch_bounds__(256) void diff_heads_norm_kernel(T* __restrict__ out, const T* __restrict__ attn,
+template <typename T, typename TA>
+__global__ __launch_bounds__(256) void diff_heads_norm_kernel(T* __restrict__ out, const TA* __restrict__ attn,
                                                               int64_t attn_stride, float lambda, float eps,
                                                               float post, int64_t pairs, int heads, int dv) {
   const int lane = threadIdx.x & (kWave - 1);
@@ -265,8 +265,8 @@ __global__ __launch_bounds__(256) void diff_heads_norm_kernel(T* __restrict__ ou
   if (th >= pairs) return;  // the whole wave
   const int64_t t = th / heads;
   const int h = static_cast<int>(th - t * heads);
-  const T* a1 = attn + t * attn_stride + static_cast<int64_t>(2 * h) * dv;
-  const T* a2 = a1 + dv;
+  const TA* a1 = attn + t * attn_stride + static_cast<int64_t>(2 * h) * dv;
+  const TA* a2 = a1 + dv;
   float ss = 0.f;
   for (int e = lane; e < dv; e += kWave) {
     const float o = to_float(a1[e]) - lambda * to_float(a2[e]);
@@ -352,17 +352,25 @@ extern "C" int kvc_head_gate(void* out, const void* x, int64_t x_stride, const v
   return kvc_check_launch("kvc_head_gate");
 }
 
-extern "C" int kvc_diff_heads_norm(void* out, const void* attn, int64_t attn_stride, float lambda, float eps, float post,
-                                   int T, int heads, int dv, int dtype, kvc_stream stream) {
+extern "C" int kvc_diff_heads_norm(void* out, const void* attn, int64_t attn_stride, int attn_dtype, float lambda,
+                                   float eps, float post, int T, int heads, int dv, int dtype, kvc_stream stream) {
   if (T < 0 || heads <= 0 || dv <= 0 || attn_stride < static_cast<int64_t>(2) * heads * dv)
     return kvc_fail("kvc_diff_heads_norm: bad sizes");
   if (out == nullptr || attn == nullptr) return kvc_fail("kvc_diff_heads_norm: null operand");
   const int64_t pairs = static_cast<int64_t>(T) * heads;
   if (pairs == 0) return 0;
   const unsigned blocks = static_cast<unsigned>((pairs + 3) / 4);
-  KVC_DISPATCH_DTYPE(dtype, Tp,
-                     hipLaunchKernelGGL(diff_heads_norm_kernel<Tp>, dim3(blocks), dim3(256), 0, S(stream),
-                                        static_cast<Tp*>(out), static_cast<const Tp*>(attn), attn_stride, lambda, eps,
-                                        post, pairs, heads, dv));
+  if (attn_dtype != dtype && attn_dtype != 0) return kvc_fail("kvc_diff_heads_norm: the maps have out's dtype or are float32");
+  if (attn_dtype == 0) {
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL((diff_heads_norm_kernel<Tp, float>), dim3(blocks), dim3(256), 0, S(stream),
+                                          static_cast<Tp*>(out), static_cast<const float*>(attn), attn_stride, lambda,
+                                          eps, post, pairs, heads, dv));
+  } else {
+    KVC_DISPATCH_DTYPE(dtype, Tp,
+                       hipLaunchKernelGGL((diff_heads_norm_kernel<Tp, Tp>), dim3(blocks), dim3(256), 0, S(stream),
+                                          static_cast<Tp*>(out), static_cast<const Tp*>(attn), attn_stride, lambda,
+                                          eps, post, pairs, heads, dv));
+  }
   return kvc_check_launch("kvc_diff_heads_norm");
 }

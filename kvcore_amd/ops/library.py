@@ -46,7 +46,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_activation": [P, P, L, I, I, P],
         "kvc_hyper_step": [P, I, P, P, I, I, P, I, P, P, F, P, P, F, I, I, I, P],
         "kvc_spread_streams": [P, P, I, I, I, P],
-        "kvc_diff_heads_norm": [P, P, L, F, F, F, I, I, I, I, P],
+        "kvc_diff_heads_norm": [P, P, L, I, F, F, F, I, I, I, I, P],
         "kvc_norm_add_norm": [P, I, P, P, I, P, F, P, F, I, I, I, P],
         "kvc_wide_qk_norm": [P, L, P, P, F, I, I, I, I, I, P],
         "kvc_head_gate": [P, P, L, P, L, I, I, I, I, I, I, P],
@@ -58,7 +58,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_rope_table": [P, P, P, P, I, I, P],
         "kvc_kv_slots": [P, P, P, P, P, I, I, I, I, P],
         "kvc_rope_kv_write": [P, P, P, P, P, I, I, P, I, I, I, I, I, I, I, I, P],
-        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, I, P],
+        "kvc_paged_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, I, I, P],
         "kvc_linear_state_scan": [P, P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, I, I, I, I, I, I, F, I, P],
         "kvc_sigmoid_power": [P, P, L, P, F, I, I, P],
         "kvc_decay_and_write_gates": [P, P, P, L, P, L, P, P, I, I, P],
@@ -83,12 +83,12 @@ def _declare(lib: ctypes.CDLL) -> None:
         "kvc_ssm_scan": [P, P, L, P, L, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
         "kvc_gated_group_rmsnorm": [P, I, P, P, L, I, P, F, I, I, I, P],
         "kvc_decode_attention": [P, P, P, P, L, P, P, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I,
-                                 F, I, P, I, P, I, P],
+                                 F, I, P, I, P, I, I, P],
         "kvc_decode_attention_waves": [I, I, I],
         "kvc_decode_attention_max_table": [I, I, I],
         "kvc_decode_attention_supported": [I, I, I, I, I],
         "kvc_prefill_attention": [P, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P, I, P, P, P, I,
-                                  P, P, I, I, P],
+                                  P, P, I, I, I, P],
         "kvc_prefill_attention_supported": [I, I, I, I, I],
         "kvc_gemm_mid_slices": [I, I],
         "kvc_gemm_mid_bf16": [P, P, P, P, P, I, I, I, L, L, I, I, I, P],
@@ -402,13 +402,15 @@ def spread_streams(streams: torch.Tensor, rows: torch.Tensor, copies: int) -> No
 def diff_heads_norm(out: torch.Tensor, attn: torch.Tensor, *, heads: int, dv: int, lam: float, eps: float,
                     post: float) -> None:
     """Rows of ``attn`` hold ``heads`` pairs of results ``[a1 | a2]`` of ``dv`` values each; ``out[t,
-    h] = (a1 - lam * a2) / sqrt(mean((a1 - lam * a2)^2) + eps) * post`` over the head's ``dv`` values."""
+    h] = (a1 - lam * a2) / sqrt(mean((a1 - lam * a2)^2) + eps) * post`` over the head's ``dv`` values.
+    ``attn`` has the dtype of ``out`` or is float32 (results that were never rounded)."""
     T = out.shape[0]
     if out.shape != (T, heads * dv) or not out.is_contiguous() or attn.shape[0] < T or attn.stride(1) != 1 \
-            or attn.shape[1] < 2 * heads * dv or attn.dtype != out.dtype:
+            or attn.shape[1] < 2 * heads * dv or attn.dtype not in (out.dtype, torch.float32):
         raise KernelError("diff_heads_norm: shapes do not match")
-    _check(load().kvc_diff_heads_norm(_dev(out, "out"), attn.data_ptr(), attn.stride(0), float(lam), float(eps),
-                                      float(post), T, heads, dv, _code(out, "out"), _stream()), "kvc_diff_heads_norm")
+    _check(load().kvc_diff_heads_norm(_dev(out, "out"), attn.data_ptr(), attn.stride(0), _code(attn, "attn"),
+                                      float(lam), float(eps), float(post), T, heads, dv, _code(out, "out"),
+                                      _stream()), "kvc_diff_heads_norm")
 
 
 def gather_rows(out: torch.Tensor, src: torch.Tensor, rows: torch.Tensor) -> None:
@@ -485,17 +487,19 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     of a value head where it differs from a key head's ``d`` (``out`` is ``[T, nh*dv]``).
     ``slopes`` (float32 ``[nh]``): ``slopes[h] * distance`` is taken off every score of head h;
     ``chunk``: a token sees only the keys of its own chunk of that many positions.  ``sinks``
-    (float32 ``[nh]``): ``exp(sinks[h])`` joins the softmax's denominator of head h."""
+    (float32 ``[nh]``): ``exp(sinks[h])`` joins the softmax's denominator of head h.  ``out`` has
+    the queries' dtype, or is float32 beside bfloat16 queries: the weighted sums unrounded (the two
+    matrix-core kernels take such an ``out`` too)."""
     if slopes is not None and (slopes.shape != (nh,) or slopes.dtype != torch.float32):
         raise KernelError("paged_attention: slopes must be float32 [nh]")
     T = out.shape[0]
     dv = d if dv is None else dv
     if out.shape != (T, nh * dv) or not out.is_contiguous():
         raise KernelError("paged_attention: out must be contiguous [T, nh*dv]")
-    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
+    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or out.dtype not in (q.dtype, torch.float32):
         raise KernelError("paged_attention: q does not fit")
     num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "paged_attention", dv)
-    if k_cache.dtype != out.dtype:
+    if k_cache.dtype != q.dtype:
         raise KernelError("paged_attention: cache dtype differs from the queries'")
     if positions.numel() < T or token_req.numel() < T:
         raise KernelError("paged_attention: per-token arrays too short")
@@ -505,7 +509,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         _dev(positions, "positions", torch.int32), _dev(token_req, "token_req", torch.int32),
         _dev(slots, "slots", torch.int32), T, nh, nkv, d, dv, page_size, num_pages, float(scale),
         int(window), None if slopes is None else _dev(slopes, "slopes"), int(chunk), _sinks(sinks, nh),
-        _code(out, "out"), _stream()), "kvc_paged_attention")
+        int(out.dtype == torch.float32 and q.dtype != torch.float32), _code(q, "q"), _stream()), "kvc_paged_attention")
 
 
 def qk_norm_rope_kv_write(qkv: torch.Tensor, k_cache: torch.Tensor,
@@ -662,13 +666,13 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
     ``part_ml`` are float32 workspaces of at least ``T*nh*nsplit*d`` and ``T*nh*nsplit*2``
     elements when ``nsplit > 1``."""
     T = out.shape[0]
-    if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
-        raise KernelError("decode_attention: out must be contiguous bfloat16 [T, nh*d]")
+    if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError("decode_attention: out must be contiguous bfloat16 (or float32) [T, nh*d]")
     need = (nh + 2 * nkv) * d if write_kv else nh * d
-    if qkv.shape[0] != T or qkv.stride(1) != 1 or qkv.shape[1] < need or qkv.dtype != out.dtype:
+    if qkv.shape[0] != T or qkv.stride(1) != 1 or qkv.shape[1] < need or qkv.dtype != torch.bfloat16:
         raise KernelError("decode_attention: qkv does not fit")
     num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "decode_attention")
-    if k_cache.dtype != out.dtype:
+    if k_cache.dtype != qkv.dtype:
         raise KernelError("decode_attention: cache dtype differs from the queries'")
     if positions.numel() < T or token_req.numel() < T:
         raise KernelError("decode_attention: per-token arrays too short")
@@ -692,7 +696,8 @@ def decode_attention(out: torch.Tensor, qkv: torch.Tensor, k_cache: torch.Tensor
         None if token_rows is None else _dev(token_rows, "token_rows", torch.int32),
         c, s_, int(rot_dim), int(bool(interleaved)),
         int(bool(write_kv)), T, nh, nkv, d, page_size, num_pages, float(scale),
-        int(window), _slopes(slopes, nh), int(chunk), _sinks(sinks, nh), int(nsplit), _stream()),
+        int(window), _slopes(slopes, nh), int(chunk), _sinks(sinks, nh), int(nsplit),
+        int(out.dtype == torch.float32), _stream()),
         "kvc_decode_attention")
 
 
@@ -714,12 +719,12 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     With ``cos`` and ``sin`` (``[T, rot_dim / 2]`` float32) the queries come unrotated and
     the kernel rotates them (``prefill_attention_rotates`` says for which shapes)."""
     T = out.shape[0]
-    if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype != torch.bfloat16:
-        raise KernelError("prefill_attention: out must be contiguous bfloat16 [T, nh*d]")
-    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != out.dtype:
+    if out.shape != (T, nh * d) or not out.is_contiguous() or out.dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError("prefill_attention: out must be contiguous bfloat16 (or float32) [T, nh*d]")
+    if q.shape[0] != T or q.stride(1) != 1 or q.shape[1] < nh * d or q.dtype != torch.bfloat16:
         raise KernelError("prefill_attention: q does not fit")
     num_pages, page_size = _check_cache(k_cache, v_cache, nkv, d, "prefill_attention")
-    if k_cache.dtype != out.dtype:
+    if k_cache.dtype != q.dtype:
         raise KernelError("prefill_attention: cache dtype differs from the queries'")
     if positions.numel() < T or q_start.numel() < num_reqs + 1 or slots.numel() < num_reqs:
         raise KernelError("prefill_attention: index arrays too short")
@@ -740,7 +745,8 @@ def prefill_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
         _dev(table, "table", torch.int32), table.shape[1], _dev(positions, "positions", torch.int32),
         _dev(q_start, "q_start", torch.int32), _dev(slots, "slots", torch.int32), T, num_reqs,
         nh, nkv, d, page_size, num_pages, float(scale), int(window), _slopes(slopes, nh), int(chunk),
-        _sinks(sinks, nh), po, pml, int(nsplit), cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved), _stream()),
+        _sinks(sinks, nh), po, pml, int(nsplit), cs, sn, int(rot_dim) if cs is not None else 0, int(interleaved),
+        int(out.dtype == torch.float32), _stream()),
         "kvc_prefill_attention")
 
 

@@ -95,6 +95,9 @@ class PagedAttention(Mixer):
     pages of that many tokens for this layer's group (None: the engine's block size)."""
 
     any_head_size = False  # a subclass whose heads need not be a multiple of 16 takes the general kernels then
+    # a subclass that joins the heads' results before anything is rounded asks the attention kernels
+    # for their float32 sums instead of results in the model's dtype
+    float32_heads = False
 
     @property
     def takes_scaled_rows(self) -> bool:  # x only goes into the qkv product
@@ -302,7 +305,10 @@ class PagedAttention(Mixer):
             rot_dim, interleaved = 0, False
         else:
             cos, sin, rot_dim, interleaved = rot.cos, rot.sin, rot.rot_dim, rot.interleaved
-        attn = ctx.buf(_sized("attn_out", self.o_size, self.shared_buffers), self.o_size)
+        if self.float32_heads:
+            attn = ctx.buf(f"attn_out_f32:{self.o_size}", self.o_size, torch.float32)
+        else:
+            attn = ctx.buf(_sized("attn_out", self.o_size, self.shared_buffers), self.o_size)
         # with a norm of the heads, or values of another size than the keys, one kernel norms,
         # rotates and writes the cache; the attention kernels then take q and the cache as they are
         prepared = not self.plain
@@ -322,7 +328,7 @@ class PagedAttention(Mixer):
             # the same scores against each plane of the values; the planes' results, each [T, heads
             # * plane size], are then laid side by side within every head
             T, m, part = ctx.num_tokens, self.v_planes, self.num_heads * self.v_plane_dim
-            parts = ctx.buffers.get(f"attn_planes:{part}", m * T, part, ctx.dtype,
+            parts = ctx.buffers.get(f"attn_planes:{part}:{attn.dtype}", m * T, part, attn.dtype,
                                     reserve=m * ctx.buffers.token_capacity)
             for c in range(m):
                 self._attend(parts[c * T: (c + 1) * T], qkv, k_cache, v_planes[c], ctx, call, group, cos, sin,
@@ -453,6 +459,9 @@ class DifferentialAttention(PagedAttention):
 
     any_head_size = True
     takes_sink = False  # the maps are joined between the attention and the output product's input
+    # where the two maps nearly cancel (lambda near one, a short window), rounding them to bfloat16
+    # first would be magnified by the head's norm: they are joined as float32 sums
+    float32_heads = True
 
     @property
     def takes_slice_sink(self) -> bool:  # float32 partial sums whatever the result's type

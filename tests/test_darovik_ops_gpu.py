@@ -149,6 +149,15 @@ def test_the_second_map_is_taken_off_and_the_head_normed(heads, dv, dtype):
     out = torch.full((T, heads * dv), float("nan"), dtype=dtype, device=DEV)
     ops.diff_heads_norm(out, gpu(rows, dtype)[:, : 2 * heads * dv], heads=heads, dv=dv, lam=lam, eps=eps, post=1 - diff)
     assert rel(out.view(T, heads, dv), want) < (2e-6 if dtype == torch.float32 else 4e-3)
+    # maps that were never rounded (float32) beside a result in the model's dtype: two maps that
+    # nearly cancel keep their difference
+    near = torch.randn(T, heads, 1, dv, generator=gen, dtype=F64).expand(T, heads, 2, dv).clone()
+    near[:, :, 1] = near[:, :, 0] / lam * (1 + 1e-3 * torch.randn(T, heads, dv, generator=gen, dtype=F64))
+    near = near.float().double()
+    want = plain.rms(near[:, :, 0] - lam * near[:, :, 1], eps) * (1 - diff)
+    out = torch.full((T, heads * dv), float("nan"), dtype=dtype, device=DEV)
+    ops.diff_heads_norm(out, gpu(near.reshape(T, -1)), heads=heads, dv=dv, lam=lam, eps=eps, post=1 - diff)
+    assert rel(out.view(T, heads, dv), want) < (2e-3 if dtype == torch.float32 else 6e-3)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
